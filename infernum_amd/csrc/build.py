@@ -46,6 +46,8 @@ CORE_SOURCES = [
     "latent.hip",
     "moe.hip",
     "seqmix.hip",
+    "linear_attention.hip",
+    "sigmoid_attention.hip",
     "sampling.hip",
     "peaks.hip",
 ]

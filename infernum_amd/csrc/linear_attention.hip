@@ -1,0 +1,191 @@
+// Gated linear attention: a recurrence per head over a state S [dim, vdim] of fp32 values with one decay per key
+// channel and token,
+//     S_t = diag(alpha_t) S_(t-1) + k_t v_t^T,      o_t = S_t^T (c q_t),      alpha = sigmoid(z)^(1/tau),
+// and what follows it: every head's o divided by its root mean square over vdim, times a weight shared by the heads,
+// times silu(gate).
+//
+//   ia_gla_scan         the recurrence token after token for the rows of every request of a step, from the request's
+//                       state slot, which it leaves moved on;
+//   ia_head_norm_gate   norm per head, weight, silu(gate), rounded once into the activations' type.
+//
+// The state of a head is kept in slices of GLA_PW value columns: slot[head][slice][n][GLA_PW], so that the workgroup
+// that owns (request, head, slice) reads and writes one stretch of memory.  log(alpha) = log_sigmoid(z) / tau and
+// every product that touches the state are fp32.
+#include "common.h"
+
+#define GLA_PW 16        // value columns of a workgroup's slice
+#define GLA_PARTS 16     // the key channels are dealt out over so many groups of threads
+#define GLA_TB 8         // tokens whose rows are staged together
+
+__host__ __device__ inline int gla_slices(int vdim) { return (vdim + GLA_PW - 1) / GLA_PW; }
+
+__device__ __forceinline__ float gla_log_sigmoid(float z) {
+  // log(1 / (1 + exp(-z))): never above zero, no overflow on either side
+  return z >= 0.f ? -log1pf(expf(-z)) : z - log1pf(expf(z));
+}
+
+// grid (heads, requests, slices), 256 threads: thread (part, p) keeps S[n][p] for n = part, part + 16, ... in registers.
+template <typename T, int KMAX>
+__global__ __launch_bounds__(256) void gla_scan_kernel(
+    const T* __restrict__ proj, int proj_stride, int q_col, int k_col, int v_col, const float* __restrict__ z,
+    int z_stride, const float* __restrict__ z_bias, float inv_tau, float q_scale, float* __restrict__ state,
+    long state_stride, float* __restrict__ out, const int* __restrict__ seq_starts, const int* __restrict__ state_slots,
+    int nh, int dim, int vdim) {
+  extern __shared__ float lds[];
+  float* qs = lds;                                   // [TB][dim]
+  float* ks = qs + GLA_TB * dim;                     // [TB][dim]
+  float* as = ks + GLA_TB * dim;                     // [TB][dim]  alpha
+  float* vs = as + GLA_TB * dim;                     // [TB][PW]
+  float* ysum = vs + GLA_TB * GLA_PW;                // [TB][PARTS][PW]
+  const int hd = blockIdx.x, s = blockIdx.y, slice = blockIdx.z;
+  const int first = seq_starts[s], count = seq_starts[s + 1] - first;
+  if (count <= 0) return;
+  const int tid = threadIdx.x;
+  const int p = tid % GLA_PW, part = tid / GLA_PW;
+  const int col = slice * GLA_PW + p;
+  const int slices = gla_slices(vdim);
+  float* S = state + (size_t)state_slots[s] * state_stride + ((size_t)hd * slices + slice) * dim * GLA_PW;
+  float reg[KMAX];
+#pragma unroll
+  for (int c = 0; c < KMAX; ++c) {
+    const int n = part + c * GLA_PARTS;
+    reg[c] = n < dim ? S[(size_t)n * GLA_PW + p] : 0.f;
+  }
+  for (int t0 = 0; t0 < count; t0 += GLA_TB) {
+    const int nt = count - t0 < GLA_TB ? count - t0 : GLA_TB;
+    __syncthreads();                                  // the block before is read to its end
+    for (int i = tid; i < nt * dim; i += 256) {
+      const int t = i / dim, n = i - t * dim;
+      const size_t row = (size_t)(first + t0 + t);
+      const T* pr = proj + row * proj_stride;
+      qs[i] = to_float(pr[q_col + hd * dim + n]) * q_scale;
+      ks[i] = to_float(pr[k_col + hd * dim + n]);
+      const float zz = z[row * z_stride + hd * dim + n] + (z_bias ? z_bias[hd * dim + n] : 0.f);
+      as[i] = expf(gla_log_sigmoid(zz) * inv_tau);
+    }
+    for (int i = tid; i < nt * GLA_PW; i += 256) {
+      const int t = i / GLA_PW, c = slice * GLA_PW + (i - t * GLA_PW);
+      vs[i] = c < vdim ? to_float(proj[(size_t)(first + t0 + t) * proj_stride + v_col + hd * vdim + c]) : 0.f;
+    }
+    __syncthreads();
+    for (int t = 0; t < nt; ++t) {
+      const float v = vs[t * GLA_PW + p];
+      const float* qt = qs + t * dim;
+      const float* kt = ks + t * dim;
+      const float* at = as + t * dim;
+      float acc = 0.f;
+#pragma unroll
+      for (int c = 0; c < KMAX; ++c) {
+        const int n = part + c * GLA_PARTS;
+        if (n < dim) {
+          reg[c] = __builtin_fmaf(at[n], reg[c], kt[n] * v);
+          acc = __builtin_fmaf(reg[c], qt[n], acc);
+        }
+      }
+      ysum[(t * GLA_PARTS + part) * GLA_PW + p] = acc;
+    }
+    __syncthreads();
+    for (int i = tid; i < nt * GLA_PW; i += 256) {
+      const int t = i / GLA_PW, pp = i - t * GLA_PW;
+      const int c = slice * GLA_PW + pp;
+      float y = ysum[(t * GLA_PARTS) * GLA_PW + pp];
+#pragma unroll
+      for (int k = 1; k < GLA_PARTS; ++k) y += ysum[(t * GLA_PARTS + k) * GLA_PW + pp];
+      if (c < vdim) out[(size_t)(first + t0 + t) * ((size_t)nh * vdim) + (size_t)hd * vdim + c] = y;
+    }
+  }
+#pragma unroll
+  for (int c = 0; c < KMAX; ++c) {
+    const int n = part + c * GLA_PARTS;
+    if (n < dim) S[(size_t)n * GLA_PW + p] = reg[c];
+  }
+}
+
+// Floats a request's slot holds for one layer run.
+extern "C" long ia_gla_state_floats(int nh, int dim, int vdim) { return (long)nh * gla_slices(vdim) * dim * GLA_PW; }
+
+// proj: rows of proj_stride values (code: their type) holding q (nh dim values from q_col), k (from k_col) and v (nh vdim
+// from v_col); z fp32 rows of z_stride values, z_bias (nullable) fp32 [nh dim]; out fp32 [N, nh vdim].
+extern "C" int ia_gla_scan(const void* proj, int code, int proj_stride, int q_col, int k_col, int v_col, const float* z,
+                           int z_stride, const float* z_bias, float tau, float q_scale, float* state, long state_stride,
+                           float* out, const int* seq_starts, const int* state_slots, int B, int nh, int dim, int vdim,
+                           hipStream_t stream) {
+  if (B == 0) return IA_OK;
+  if (!proj || !z || !state || !out || !seq_starts || !state_slots || B < 0 || nh <= 0 || dim <= 0 || vdim <= 0 ||
+      !(tau > 0.f) || q_col < 0 || k_col < 0 || v_col < 0 || proj_stride < q_col + nh * dim ||
+      proj_stride < k_col + nh * dim || proj_stride < v_col + nh * vdim || z_stride < nh * dim ||
+      state_stride < ia_gla_state_floats(nh, dim, vdim))
+    return IA_ERR_BAD_ARG;
+  const int per = (dim + GLA_PARTS - 1) / GLA_PARTS;
+  const int slices = gla_slices(vdim);
+  if (per > 32 || B > 65535 || slices > 65535) return IA_ERR_UNSUPPORTED;
+  const dim3 grid((unsigned)nh, (unsigned)B, (unsigned)slices);
+  const size_t lds = sizeof(float) * ((size_t)3 * GLA_TB * dim + GLA_TB * GLA_PW + (size_t)GLA_TB * GLA_PARTS * GLA_PW);
+  if (lds > 64 * 1024) return IA_ERR_UNSUPPORTED;
+#define IA_GLA(T, KM)                                                                                                  \
+  gla_scan_kernel<T, KM><<<grid, 256, lds, stream>>>((const T*)proj, proj_stride, q_col, k_col, v_col, z, z_stride,    \
+                                                     z_bias, 1.0f / tau, q_scale, state, state_stride, out, seq_starts, \
+                                                     state_slots, nh, dim, vdim)
+#define IA_GLA_K(T)                       \
+  do {                                    \
+    if (per <= 4) IA_GLA(T, 4);           \
+    else if (per <= 8) IA_GLA(T, 8);      \
+    else if (per <= 16) IA_GLA(T, 16);    \
+    else IA_GLA(T, 32);                   \
+  } while (0)
+  if (code == IA_F32) IA_GLA_K(float);
+  else if (code == IA_BF16) IA_GLA_K(bf16_t);
+  else return IA_ERR_BAD_ARG;
+#undef IA_GLA_K
+#undef IA_GLA
+  IA_LAUNCH_CHECK();
+  return IA_OK;
+}
+
+// One wave per (token, head): y = o / sqrt(mean(o^2) + eps) * w * silu(gate), o fp32 [N, nh vdim], w fp32 [vdim],
+// gate rows of gate_stride values in the activations' type (the head's vdim values from gate_col + head * vdim).
+template <typename T>
+__global__ __launch_bounds__(256) void head_norm_gate_kernel(const float* __restrict__ o, const T* __restrict__ gate,
+                                                             int gate_stride, int gate_col, const float* __restrict__ w,
+                                                             T* __restrict__ y, long pairs, int nh, int vdim, float eps) {
+  const long pair = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (pair >= pairs) return;
+  const int lane = threadIdx.x & 63;
+  const long n = pair / nh;
+  const int hd = (int)(pair - n * nh);
+  const float* orow = o + (size_t)pair * vdim;
+  float ss = 0.f;
+  for (int i = lane; i < vdim; i += 64) ss = fmaf(orow[i], orow[i], ss);
+  ss = wave_sum(ss);
+  const float inv = 1.0f / sqrtf(ss / (float)vdim + eps);
+  const T* grow = gate + (size_t)n * gate_stride + gate_col + (size_t)hd * vdim;
+  for (int i = lane; i < vdim; i += 64) {
+    const float g = to_float(grow[i]);
+    y[(size_t)pair * vdim + i] = from_float<T>(orow[i] * inv * w[i] * (g / (1.0f + expf(-g))));
+  }
+}
+
+extern "C" int ia_head_norm_gate(const float* o, const void* gate, int code, int gate_stride, int gate_col,
+                                 const float* w, void* y, int N, int nh, int vdim, float eps, hipStream_t stream) {
+  if (N < 0 || nh <= 0 || vdim <= 0 || !(eps > 0.f) || gate_col < 0 || gate_stride < gate_col + nh * vdim)
+    return IA_ERR_BAD_ARG;
+  if (N == 0) return IA_OK;
+  if (!o || !gate || !w || !y) return IA_ERR_BAD_ARG;
+  const long pairs = (long)N * nh;
+  const long blocks = (pairs + 3) / 4;
+  if (blocks > 0x7fffffffL) return IA_ERR_UNSUPPORTED;
+  if (code == IA_F32)
+    head_norm_gate_kernel<float><<<(unsigned)blocks, 256, 0, stream>>>(o, (const float*)gate, gate_stride, gate_col, w,
+                                                                       (float*)y, pairs, nh, vdim, eps);
+  else if (code == IA_BF16)
+    head_norm_gate_kernel<bf16_t><<<(unsigned)blocks, 256, 0, stream>>>(o, (const bf16_t*)gate, gate_stride, gate_col, w,
+                                                                        (bf16_t*)y, pairs, nh, vdim, eps);
+  else
+    return IA_ERR_BAD_ARG;
+  IA_LAUNCH_CHECK();
+  return IA_OK;
+}
+
+#include "op_call.h"
+IA_OP(ia_gla_scan)
+IA_OP(ia_head_norm_gate)

@@ -388,6 +388,167 @@ extern "C" int ia_moe_scatter(const void* o, const int* perm, const float* weigh
   return IA_OK;
 }
 
+// ---- experts without a gate, and a router whose choice and weights go by different numbers ----
+//   ia_router_softmax_topk   s = softmax(z) over all experts; the `top` largest of s + correction are chosen (the
+//                            lowest index among equals); the weights are the chosen s over their sum (+ 1e-20);
+//   ia_moe_up                per expert, over its pairs' tokens: y = act(Wu x), Wu [E, ff, W]; act by the codes of
+//                            ia_activation (2: the erf GELU, 3: the square of relu).
+__device__ __forceinline__ float moe_act(float z, int act) {
+  if (act == 3) { const float r = fmaxf(z, 0.f); return r * r; }
+  if (act == 2) return 0.5f * z * (1.0f + erff(z * 0.7071067811865476f));
+  if (act == 1) return 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+  return z;
+}
+
+__global__ __launch_bounds__(256) void router_softmax_topk_kernel(const float* __restrict__ logits,
+                                                                  const void* __restrict__ corr, int corr_dtype,
+                                                                  int* __restrict__ ids, float* __restrict__ weights,
+                                                                  int N, int E, int top) {
+  const int n = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+  if (n >= N) return;
+  const float* z = logits + (size_t)n * E;
+  float s[RT_PER_LANE], v[RT_PER_LANE];
+  unsigned taken = 0u;
+  float zmax = -INFINITY;
+#pragma unroll
+  for (int c = 0; c < RT_PER_LANE; ++c) {
+    const int e = lane + 64 * c;
+    s[c] = e < E ? z[e] : -INFINITY;
+    zmax = fmaxf(zmax, s[c]);
+    if (e >= E) taken |= 1u << c;
+  }
+  zmax = wave_max(zmax);
+  float total = 0.f;
+#pragma unroll
+  for (int c = 0; c < RT_PER_LANE; ++c) {
+    s[c] = (lane + 64 * c) < E ? expf(s[c] - zmax) : 0.f;
+    total += s[c];
+  }
+  total = wave_sum(total);
+  const float inv_total = 1.0f / total;
+#pragma unroll
+  for (int c = 0; c < RT_PER_LANE; ++c) {
+    const int e = lane + 64 * c;
+    s[c] *= inv_total;
+    v[c] = e < E ? s[c] + (corr ? load_as_float(corr, corr_dtype, e) : 0.f) : -INFINITY;
+  }
+  float sum = 0.f;
+  for (int k = 0; k < top; ++k) {
+    float best_v = -INFINITY, best_s = 0.f;
+    int best_e = 0x7fffffff;
+#pragma unroll
+    for (int c = 0; c < RT_PER_LANE; ++c) {
+      const bool free_ = !((taken >> c) & 1u);
+      const float x = (v[c] == v[c]) ? v[c] : -INFINITY;
+      if (free_ && (best_e == 0x7fffffff || x > best_v)) { best_v = x; best_e = lane + 64 * c; best_s = s[c]; }
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+      const float ov = __shfl_xor(best_v, o, IA_WAVE), os = __shfl_xor(best_s, o, IA_WAVE);
+      const int oe = __shfl_xor(best_e, o, IA_WAVE);
+      if (oe != 0x7fffffff && (best_e == 0x7fffffff || ov > best_v || (ov == best_v && oe < best_e))) {
+        best_v = ov;
+        best_e = oe;
+        best_s = os;
+      }
+    }
+    if ((best_e & 63) == lane) taken |= 1u << (best_e >> 6);
+    sum += best_s;
+    if (lane == 0) {
+      ids[(size_t)n * top + k] = best_e;
+      weights[(size_t)n * top + k] = best_s;
+    }
+  }
+  const float inv = 1.0f / (sum + 1e-20f);
+  if (lane == 0)
+    for (int k = 0; k < top; ++k) weights[(size_t)n * top + k] *= inv;
+}
+
+extern "C" int ia_router_softmax_topk(const float* logits, const void* corr, int corr_dtype, int* ids, float* weights,
+                                      int N, int E, int top, hipStream_t stream) {
+  if (N < 0 || E <= 0 || top <= 0 || top > E || !logits || !ids || !weights) return IA_ERR_BAD_ARG;
+  if (E > 64 * RT_PER_LANE) return IA_ERR_UNSUPPORTED;
+  if (N == 0) return IA_OK;
+  router_softmax_topk_kernel<<<(N + 3) / 4, 256, 0, stream>>>(logits, corr, corr_dtype, ids, weights, N, E, top);
+  IA_LAUNCH_CHECK();
+  return IA_OK;
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void moe_up_kernel(const T* __restrict__ x, const T* __restrict__ Wu, T* __restrict__ y,
+                                                     const int* __restrict__ offsets, const int* __restrict__ perm,
+                                                     int E, int top, int W, int ff, int act) {
+  __shared__ TileFmaLds lds;
+  int e, first, last;
+  if (!moe_tile(offsets, E, blockIdx.y, e, first, last)) return;
+  const int n0 = blockIdx.x * TF_T;
+  const int lr = threadIdx.x >> 2;
+  const T* a_row = (first + lr < last) ? x + (size_t)(perm[first + lr] / top) * W : nullptr;
+  const T* w_row = (n0 + lr < ff) ? Wu + ((size_t)e * ff + n0 + lr) * W : nullptr;
+  tile_64(a_row, w_row, W, lds, [&](int i, int j0, const float* v) {
+    const int p = first + i;
+    if (p >= last) return;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int c = n0 + j0 + j;
+      // the product is rounded as a stored tensor would be, then the activation in fp32
+      if (c < ff) y[(size_t)p * ff + c] = from_float<T>(moe_act(to_float(from_float<T>(v[j])), act));
+    }
+  });
+}
+
+template <int BM, int BN>
+__global__ __launch_bounds__(BN == 256 ? 512 : 256) void moe_up_big_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ Wu,
+                                                              bf16_t* __restrict__ y, const int* __restrict__ offsets,
+                                                              const int* __restrict__ perm, int E, int top, int W,
+                                                              int ff, int act) {
+  __shared__ TileBigLds<BM, BN> lds;
+  int e, first, last;
+  if (!moe_tile(offsets, E, blockIdx.y, e, first, last, BM)) return;
+  const int n0 = blockIdx.x * BN;
+  tile_mfma_big<BM, BN>(
+      [&](int r) { return x + (size_t)(perm[first + r] / top) * W; },
+      [&](int r) { return Wu + ((size_t)e * ff + n0 + r) * W; }, last - first, ff - n0, W, lds,
+      [&](int i, int j0, const float* v) {
+        const int p = first + i;
+        if (p >= last) return;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const int c = n0 + j0 + j;
+          if (c < ff) y[(size_t)p * ff + c] = from_float<bf16_t>(moe_act(to_float(from_float<bf16_t>(v[j])), act));
+        }
+      });
+}
+
+extern "C" int ia_moe_up(const void* x, const void* Wu, void* y, const int* offsets, const int* perm, int dtype, int P,
+                         int E, int top, int W, int ff, int act, hipStream_t stream) {
+  if (P < 0 || E <= 0 || top <= 0 || W <= 0 || ff <= 0 || act < 0 || act > 3) return IA_ERR_BAD_ARG;
+  if (P == 0) return IA_OK;
+  dim3 grid((ff + TF_T - 1) / TF_T, (P + TF_T - 1) / TF_T + E);
+  if (grid.y > 65535u) return IA_ERR_UNSUPPORTED;
+  if (dtype == IA_F32)
+    moe_up_kernel<float><<<grid, 256, 0, stream>>>((const float*)x, (const float*)Wu, (float*)y, offsets, perm, E, top,
+                                                   W, ff, act);
+  else if (dtype == IA_BF16 && tile_rows_aligned(x, W) && tile_rows_aligned(Wu, W)) {
+    const int bm = moe_tile_rows(P, E);
+    const int bn = bm == 128 ? 256 : TB_N;
+    dim3 big((ff + bn - 1) / bn, (P + bm - 1) / bm + E);
+    if (big.y > 65535u) return IA_ERR_UNSUPPORTED;
+    if (bm == 128)
+      moe_up_big_kernel<128, 256><<<big, 512, 0, stream>>>((const bf16_t*)x, (const bf16_t*)Wu, (bf16_t*)y, offsets, perm,
+                                                           E, top, W, ff, act);
+    else
+      moe_up_big_kernel<32, TB_N><<<big, 256, 0, stream>>>((const bf16_t*)x, (const bf16_t*)Wu, (bf16_t*)y, offsets, perm,
+                                                          E, top, W, ff, act);
+  } else if (dtype == IA_BF16)
+    moe_up_kernel<bf16_t><<<grid, 256, 0, stream>>>((const bf16_t*)x, (const bf16_t*)Wu, (bf16_t*)y, offsets, perm, E,
+                                                    top, W, ff, act);
+  else
+    return IA_ERR_BAD_ARG;
+  IA_LAUNCH_CHECK();
+  return IA_OK;
+}
+
 #include "op_call.h"
 IA_OP(ia_router_topk)
 IA_OP(ia_moe_sort)
@@ -396,3 +557,5 @@ IA_OP(ia_moe_down)
 IA_OP(ia_moe_gather)
 IA_OP(ia_moe_glu)
 IA_OP(ia_moe_scatter)
+IA_OP(ia_router_softmax_topk)
+IA_OP(ia_moe_up)

@@ -154,5 +154,147 @@ extern "C" int ia_norm_add(float* h, const void* delta, int delta_dtype, int spl
   return IA_OK;
 }
 
+// ---- the same with a gate on the branch, and optionally the next sublayer's norm behind the add ----
+//   d = sum_k delta[k][n] * sigmoid(gate[n] + gate_bias)   (fp32; the gate's logits in fp32 or the activations' type)
+//   h[n] += d / sqrt(mean(d^2) + eps) * w
+//   x[n] = h[n] / sqrt(mean(h[n]^2) + eps) * w_next   (with w_next; without it x[n] = h[n]; x may be absent)
+// One workgroup a row, the row's values in registers (rows above NB_NT * NB_KEEP values are read again).
+template <typename TD, typename TG, typename TX>
+__global__ __launch_bounds__(NB_NT) void gated_norm_add_kernel(float* __restrict__ h, const TD* __restrict__ delta,
+                                                               int splits, size_t split_stride,
+                                                               const TG* __restrict__ gate, int gate_stride,
+                                                               const float* __restrict__ gate_bias,
+                                                               const void* __restrict__ w, int w_dtype,
+                                                               const void* __restrict__ w_next, int w_next_dtype,
+                                                               TX* __restrict__ x, int H, float eps) {
+  __shared__ float red[NB_NT / 64];
+  const int row = blockIdx.x;
+  const TD* dr = delta + (size_t)row * H;
+  const TG* gr = gate ? gate + (size_t)row * gate_stride : nullptr;
+  float* hr = h + (size_t)row * H;
+  auto gated = [&](int i) {
+    float d = load_split_sum(dr + i, splits, split_stride);
+    if (gr) {
+      const float z = to_float(gr[i]) + (gate_bias ? gate_bias[i] : 0.f);
+      d *= 1.0f / (1.0f + expf(-z));
+    }
+    return d;
+  };
+  float keep[NB_KEEP];
+  float ss = 0.f;
+#pragma unroll
+  for (int c = 0; c < NB_KEEP; ++c) {
+    const int i = threadIdx.x + c * NB_NT;
+    keep[c] = 0.f;
+    if (i < H) {
+      keep[c] = gated(i);
+      ss = fmaf(keep[c], keep[c], ss);
+    }
+  }
+  for (int i = threadIdx.x + NB_KEEP * NB_NT; i < H; i += NB_NT) {
+    const float d = gated(i);
+    ss = fmaf(d, d, ss);
+  }
+  ss = block_sum<NB_NT>(ss, red);
+  const float inv = 1.0f / sqrtf(ss / (float)H + eps);
+  float s2 = 0.f;
+#pragma unroll
+  for (int c = 0; c < NB_KEEP; ++c) {
+    const int i = threadIdx.x + c * NB_NT;
+    if (i < H) {
+      keep[c] = hr[i] + keep[c] * inv * load_as_float(w, w_dtype, i);
+      hr[i] = keep[c];
+      s2 = fmaf(keep[c], keep[c], s2);
+    }
+  }
+  for (int i = threadIdx.x + NB_KEEP * NB_NT; i < H; i += NB_NT) {
+    const float s = hr[i] + gated(i) * inv * load_as_float(w, w_dtype, i);
+    hr[i] = s;
+    s2 = fmaf(s, s, s2);
+  }
+  if (!x) return;
+  float inv2 = 1.0f;
+  if (w_next) {
+    s2 = block_sum<NB_NT>(s2, red);
+    inv2 = 1.0f / sqrtf(s2 / (float)H + eps);
+  }
+#pragma unroll
+  for (int c = 0; c < NB_KEEP; ++c) {
+    const int i = threadIdx.x + c * NB_NT;
+    if (i < H) x[(size_t)row * H + i] = from_float<TX>(w_next ? keep[c] * inv2 * load_as_float(w_next, w_next_dtype, i) : keep[c]);
+  }
+  for (int i = threadIdx.x + NB_KEEP * NB_NT; i < H; i += NB_NT)
+    x[(size_t)row * H + i] = from_float<TX>(w_next ? hr[i] * inv2 * load_as_float(w_next, w_next_dtype, i) : hr[i]);
+}
+
+template <typename TD, typename TX>
+static int launch_gated_norm_add(float* h, const void* delta, int splits, size_t stride, const void* gate, int gate_dtype,
+                                 int gate_stride, const float* gate_bias, const void* w, int w_dtype, const void* w_next,
+                                 int w_next_dtype, void* x, int N, int H, float eps, hipStream_t stream) {
+  if (gate_dtype == IA_F32)
+    gated_norm_add_kernel<TD, float, TX><<<N, NB_NT, 0, stream>>>(h, (const TD*)delta, splits, stride, (const float*)gate,
+                                                                  gate_stride, gate_bias, w, w_dtype, w_next, w_next_dtype,
+                                                                  (TX*)x, H, eps);
+  else if (gate_dtype == IA_BF16)
+    gated_norm_add_kernel<TD, bf16_t, TX><<<N, NB_NT, 0, stream>>>(h, (const TD*)delta, splits, stride, (const bf16_t*)gate,
+                                                                   gate_stride, gate_bias, w, w_dtype, w_next, w_next_dtype,
+                                                                   (TX*)x, H, eps);
+  else
+    return IA_ERR_BAD_ARG;
+  return IA_OK;
+}
+
+// delta [splits, delta_rows, H] of delta_dtype; gate (nullable) [N, >= H] rows of gate_stride values of gate_dtype;
+// gate_bias (nullable) fp32 [H]; w_next (nullable): the weight of the norm that follows the add; x (nullable) of act_dtype.
+extern "C" int ia_gated_norm_add(float* h, const void* delta, int delta_dtype, int splits, int delta_rows, const void* gate,
+                                 int gate_dtype, int gate_stride, const float* gate_bias, const void* w, int w_dtype,
+                                 const void* w_next, int w_next_dtype, void* x, int act_dtype, int N, int H, float eps,
+                                 hipStream_t stream) {
+  if (N < 0 || H <= 0 || !(eps > 0.f) || !delta || !h || !w || splits < 1 || delta_rows < N || (gate && gate_stride < H))
+    return IA_ERR_BAD_ARG;
+  if (N == 0) return IA_OK;
+  const size_t stride = (size_t)delta_rows * H;
+  int rc;
+  if (delta_dtype == IA_F32 && act_dtype == IA_F32)
+    rc = launch_gated_norm_add<float, float>(h, delta, splits, stride, gate, gate_dtype, gate_stride, gate_bias, w, w_dtype,
+                                             w_next, w_next_dtype, x, N, H, eps, stream);
+  else if (delta_dtype == IA_BF16 && act_dtype == IA_BF16)
+    rc = launch_gated_norm_add<bf16_t, bf16_t>(h, delta, splits, stride, gate, gate_dtype, gate_stride, gate_bias, w,
+                                               w_dtype, w_next, w_next_dtype, x, N, H, eps, stream);
+  else if (delta_dtype == IA_F32 && act_dtype == IA_BF16)
+    rc = launch_gated_norm_add<float, bf16_t>(h, delta, splits, stride, gate, gate_dtype, gate_stride, gate_bias, w,
+                                              w_dtype, w_next, w_next_dtype, x, N, H, eps, stream);
+  else
+    return IA_ERR_BAD_ARG;
+  if (rc != IA_OK) return rc;
+  IA_LAUNCH_CHECK();
+  return IA_OK;
+}
+
+// h[n, :] += table[index[n], :] (fp32 sums; the table in fp32 or bfloat16): a learned vector per position.  An index
+// outside the table leaves NaN, never a stray read.
+__global__ __launch_bounds__(256) void add_rows_kernel(float* __restrict__ h, const void* __restrict__ table, int dtype,
+                                                       const int* __restrict__ index, int H, int rows) {
+  const int n = blockIdx.x;
+  const int r = index[n];
+  float* hr = h + (size_t)n * H;
+  if ((unsigned)r >= (unsigned)rows) {
+    for (int i = threadIdx.x; i < H; i += 256) hr[i] = __uint_as_float(0x7fc00000u);
+    return;
+  }
+  for (int i = threadIdx.x; i < H; i += 256) hr[i] += load_as_float(table, dtype, (size_t)r * H + i);
+}
+
+extern "C" int ia_add_rows(float* h, const void* table, int dtype, const int* index, int N, int H, int rows,
+                           hipStream_t stream) {
+  if (N < 0 || H <= 0 || rows <= 0 || !h || !table || !index || (dtype != IA_F32 && dtype != IA_BF16)) return IA_ERR_BAD_ARG;
+  if (N == 0) return IA_OK;
+  add_rows_kernel<<<N, 256, 0, stream>>>(h, table, dtype, index, H, rows);
+  IA_LAUNCH_CHECK();
+  return IA_OK;
+}
+
 #include "op_call.h"
 IA_OP(ia_norm_add)
+IA_OP(ia_gated_norm_add)
+IA_OP(ia_add_rows)

@@ -217,11 +217,11 @@ def norm_add(h: torch.Tensor, delta, weight: torch.Tensor, eps: float, x: Option
     return h
 
 
-ACTIVATIONS = {"gelu_tanh": 1}
+ACTIVATIONS = {"gelu_tanh": 1, "gelu": 2, "relu_squared": 3}
 
 
 def activation(x: torch.Tensor, kind: str, out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """out = act(x) element by element in fp32 (in place without ``out``).  Kinds: gelu_tanh."""
+    """out = act(x) element by element in fp32 (in place without ``out``).  Kinds: gelu_tanh, gelu (the erf form), relu_squared."""
     out = x if out is None else out
     _dev(x, out)
     _need(kind in ACTIVATIONS, f"activation: unknown kind {kind!r}; known: {sorted(ACTIVATIONS)}")
@@ -1155,6 +1155,225 @@ def softcap(logits: torch.Tensor, cap: float) -> torch.Tensor:
           "softcap: logits fp32 [R, V], cap positive")
     _ok(_core().ia_softcap(_p(logits), logits.shape[0], logits.shape[1], ctypes.c_float(cap), _stream()), "softcap")
     return logits
+
+
+def scale_(x: torch.Tensor, s: float) -> torch.Tensor:
+    """x [R, C] fp32 <- x * s, in place."""
+    _need(x.is_cuda and x.dtype == torch.float32 and x.is_contiguous() and x.dim() == 2, "scale_: x fp32 [R, C]")
+    _ok(_core().ia_scale(_p(x), x.shape[0], x.shape[1], ctypes.c_float(s), _stream()), "scale_")
+    return x
+
+
+# ------------------------------------------------- gated branches, linear attention, attention with sigmoid weights
+def add_rows(h: torch.Tensor, table: torch.Tensor, index: torch.Tensor) -> torch.Tensor:
+    """h [N, H] fp32 += table[index[n]] row by row (a learned vector per position); an index outside the table
+    leaves NaN."""
+    _dev(h, table, index)
+    N, H = h.shape
+    _need(h.dtype == torch.float32 and table.dim() == 2 and table.shape[1] == H and table.dtype in DTYPE_CODE,
+          "add_rows: h fp32 [N, H], table [rows, H]")
+    _i32(index, N, "add_rows index")
+    _ok(_core().ia_add_rows(_p(h), _p(table), DTYPE_CODE[table.dtype], _p(index), N, H, table.shape[0], _stream()),
+        "add_rows")
+    return h
+
+
+def gated_norm_add(h: torch.Tensor, delta, gate: Optional[torch.Tensor], gate_bias: Optional[torch.Tensor],
+                   weight: torch.Tensor, eps: float, next_weight: Optional[torch.Tensor] = None,
+                   x: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """d = delta * sigmoid(gate + gate_bias);  h += d * rsqrt(mean(d^2) + eps) * weight  (fp32, in place).  ``delta``: a
+    tensor of h's shape in the activations' dtype or a :class:`SplitSum`; ``gate``: rows of at least H values (fp32 or
+    the activations' dtype) or None for no gate; ``x`` (optional, h's shape in the activations' dtype) receives
+    rms_norm(h) * next_weight, or the new h itself without ``next_weight``."""
+    split = isinstance(delta, SplitSum)
+    d = delta.parts if split else delta
+    _dev(h, d, weight, x, gate_bias, next_weight)
+    _need(h.dtype == torch.float32 and h.dim() == 2, "gated_norm_add: h must be fp32 [N, H]")
+    N, H = h.shape
+    splits, d_rows = 1, N
+    if split:
+        _need(d.shape[1] >= N and d.shape[2] == H, "gated_norm_add: partial sums must be [S, >= N, H]")
+        splits, d_rows = d.shape[0], d.shape[1]
+    else:
+        _need(d is not None and d.dtype in DTYPE_CODE and tuple(d.shape) == (N, H), "gated_norm_add: delta of h's shape")
+    if gate is not None:
+        _rows(gate, H, "gated_norm_add gate")
+        _need(gate.shape[0] >= N, "gated_norm_add: a gate row per row of h")
+    _f32(gate_bias, H, "gated_norm_add gate bias")
+    for wt in (weight, next_weight):
+        _need(wt is None or (wt.dtype in DTYPE_CODE and wt.numel() == H), f"gated_norm_add: weights of {H} values")
+    act = x.dtype if x is not None else (torch.bfloat16 if d.dtype == torch.bfloat16 else torch.float32)
+    if x is not None:
+        _need(x.dtype in DTYPE_CODE and tuple(x.shape) == (N, H) and (split or x.dtype == d.dtype),
+              "gated_norm_add: x of h's shape in the activations' dtype")
+    _ok(_core().ia_gated_norm_add(
+        _p(h), _p(d), DTYPE_CODE[d.dtype], splits, d_rows, _p(gate), DTYPE_CODE[gate.dtype] if gate is not None else 0,
+        int(gate.stride(0)) if gate is not None else 0, _p(gate_bias), _p(weight), DTYPE_CODE[weight.dtype],
+        _p(next_weight), DTYPE_CODE[next_weight.dtype] if next_weight is not None else 0, _p(x), DTYPE_CODE[act], N, H,
+        ctypes.c_float(eps), _stream()), "gated_norm_add")
+    return h
+
+
+def router_softmax_topk(logits: torch.Tensor, correction: Optional[torch.Tensor], top: int):
+    """-> (ids int32 [N, top], weights fp32 [N, top]): s = softmax(logits) over all experts; the ``top`` largest of
+    s + correction are chosen (the lowest index among equals); the weights are the chosen s over their sum."""
+    _dev(logits, correction)
+    _need(logits.dtype == torch.float32 and logits.dim() == 2, "router_softmax_topk: fp32 logits [N, E]")
+    N, E = logits.shape
+    _need(0 < top <= E, f"router_softmax_topk: top must be 1 .. {E}")
+    _need(correction is None or (correction.dtype in DTYPE_CODE and correction.numel() == E),
+          f"router_softmax_topk: {E} corrections")
+    ids = torch.empty((N, top), dtype=torch.int32, device=logits.device)
+    weights = torch.empty((N, top), dtype=torch.float32, device=logits.device)
+    _ok(_core().ia_router_softmax_topk(_p(logits), _p(correction),
+                                       DTYPE_CODE[correction.dtype] if correction is not None else 0, _p(ids),
+                                       _p(weights), N, E, top, _stream()), "router_softmax_topk")
+    return ids, weights
+
+
+def moe_plain_experts(x: torch.Tensor, ids: torch.Tensor, weights: torch.Tensor, w_up: torch.Tensor,
+                      w_down: torch.Tensor, act: str, parts: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """The chosen experts of every token, each down(act(up x)) without a gate: w_up [E, ff, W], w_down [E, W, ff].
+    Fills parts[:top] of fp32 ``parts`` [>= top, N, W], each already times its routing weight, and returns parts."""
+    _dev(x, ids, weights, w_up, w_down, parts)
+    N, W = x.shape
+    E, ff, _ = w_up.shape
+    top = ids.shape[1]
+    _need(act in ACTIVATIONS, f"moe: unknown activation {act!r}")
+    _need(x.dtype in DTYPE_CODE and w_up.dtype == x.dtype and w_down.dtype == x.dtype, "moe: one dtype")
+    _need(tuple(w_up.shape) == (E, ff, W) and tuple(w_down.shape) == (E, W, ff), "moe: weights' shapes")
+    _need(ids.dtype == torch.int32 and tuple(ids.shape) == (N, top) and weights.dtype == torch.float32
+          and tuple(weights.shape) == (N, top), "moe: ids int32 and weights fp32 [N, top]")
+    if parts is None:
+        parts = torch.empty((top, N, W), dtype=torch.float32, device=x.device)
+    _need(parts.dtype == torch.float32 and parts.dim() == 3 and parts.shape[0] >= top and tuple(parts.shape[1:]) == (N, W),
+          "moe: parts fp32 [>= top, N, W]")
+    P = N * top
+    offsets = torch.empty(E + 1, dtype=torch.int32, device=x.device)
+    perm = torch.empty(max(P, 1), dtype=torch.int32, device=x.device)
+    y = torch.empty((max(P, 1), ff), dtype=x.dtype, device=x.device)
+    code = DTYPE_CODE[x.dtype]
+    _ok(_core().ia_moe_sort(_p(ids), _p(offsets), _p(perm), P, E, _stream()), "moe_sort")
+    if moe_grouped_rows(N, E, top, W, ff, x.dtype):
+        xs = torch.empty((P, W), dtype=x.dtype, device=x.device)
+        _ok(_core().ia_moe_gather(_p(x), _p(perm), _p(xs), P, top, W, _stream()), "moe_gather")
+        gemm_mfma_grouped(xs, w_up, offsets, y)
+        activation(y, act)
+        gemm_mfma_grouped(y, w_down, offsets, xs)
+        _ok(_core().ia_moe_scatter(_p(xs), _p(perm), _p(weights), _p(parts), N, top, W, _stream()), "moe_scatter")
+        return parts
+    _ok(_core().ia_moe_up(_p(x), _p(w_up), _p(y), _p(offsets), _p(perm), code, P, E, top, W, ff, ACTIVATIONS[act],
+                          _stream()), "moe_up")
+    _ok(_core().ia_moe_down(_p(y), _p(w_down), _p(parts), _p(weights), _p(offsets), _p(perm), code, N, E, top, W, ff,
+                            _stream()), "moe_down")
+    return parts
+
+
+def gla_state_floats(nh: int, dim: int, vdim: int) -> int:
+    """Floats of a request's state for one run of a gated-linear-attention layer (the heads' S in the kernel's slices)."""
+    PW = 16
+    return nh * ((vdim + PW - 1) // PW) * dim * PW
+
+
+def gla_scan(proj: torch.Tensor, q_col: int, k_col: int, v_col: int, z: torch.Tensor, z_bias: Optional[torch.Tensor],
+             tau: float, q_scale: float, state: torch.Tensor, out: torch.Tensor, seq_starts: torch.Tensor,
+             state_slots: torch.Tensor, nh: int, dim: int, vdim: int) -> torch.Tensor:
+    """Per request and head over the request's rows in order: alpha = sigmoid(z + z_bias)^(1/tau) per key channel,
+    S <- diag(alpha) S + k v^T, out = S^T (q_scale q).  ``proj`` rows hold q and k (nh dim values from q_col, k_col)
+    and v (nh vdim from v_col); ``z`` fp32 [N, nh dim]; ``state`` [slots, >= gla_state_floats] fp32 is read and left
+    moved on; ``out`` fp32 [N, nh vdim]."""
+    N, B = proj.shape[0], state_slots.numel()
+    _rows(proj, max(q_col + nh * dim, k_col + nh * dim, v_col + nh * vdim), "gla_scan rows")
+    _need(z.is_cuda and z.dtype == torch.float32 and z.dim() == 2 and z.stride(1) == 1 and z.shape[1] >= nh * dim
+          and z.shape[0] == N, "gla_scan: z fp32 [N, nh dim]")
+    _f32(z_bias, nh * dim, "gla_scan bias")
+    _need(out.is_cuda and out.dtype == torch.float32 and out.is_contiguous() and tuple(out.shape) == (N, nh * vdim),
+          "gla_scan: out [N, nh vdim] fp32")
+    _i32(seq_starts, B + 1, "gla_scan seq_starts")
+    _i32(state_slots, B, "gla_scan state_slots")
+    stride = _state_rows(state, gla_state_floats(nh, dim, vdim), "gla_scan")
+    _ok(_core().ia_gla_scan(_p(proj), DTYPE_CODE[proj.dtype], int(proj.stride(0)), q_col, k_col, v_col, _p(z),
+                            int(z.stride(0)), _p(z_bias), ctypes.c_float(tau), ctypes.c_float(q_scale), _p(state),
+                            ctypes.c_long(stride), _p(out), _p(seq_starts), _p(state_slots), B, nh, dim, vdim, _stream()),
+        "gla_scan")
+    return out
+
+
+def head_norm_gate(o: torch.Tensor, gate: torch.Tensor, gate_col: int, w: torch.Tensor, eps: float, nh: int, vdim: int,
+                   out: torch.Tensor) -> torch.Tensor:
+    """out = o / sqrt(mean(o^2) + eps) * w * silu(gate) with the mean over each head's vdim values: o fp32 [N, nh vdim],
+    w fp32 [vdim] shared by the heads, gate rows holding nh vdim values from gate_col on."""
+    N = o.shape[0]
+    _need(o.is_cuda and o.dtype == torch.float32 and o.is_contiguous() and tuple(o.shape) == (N, nh * vdim),
+          "head_norm_gate: o [N, nh vdim] fp32")
+    _rows(gate, gate_col + nh * vdim, "head_norm_gate gate")
+    _f32(w, vdim, "head_norm_gate weight")
+    _need(out.is_cuda and out.is_contiguous() and tuple(out.shape) == (N, nh * vdim) and out.dtype == gate.dtype
+          and gate.shape[0] == N, "head_norm_gate: out [N, nh vdim] of the gate's dtype")
+    _ok(_core().ia_head_norm_gate(_p(o), _p(gate), DTYPE_CODE[gate.dtype], int(gate.stride(0)), gate_col, _p(w), _p(out),
+                                  N, nh, vdim, ctypes.c_float(eps), _stream()), "head_norm_gate")
+    return out
+
+
+def sigattn_prepare(proj: torch.Tensor, bq, bk, bv, wq: torch.Tensor, wk: Optional[torch.Tensor], eps: float,
+                    temp_coef: float, temp_every: int, positions: torch.Tensor, slots: Optional[torch.Tensor],
+                    q_out: torch.Tensor, k_pages: Optional[torch.Tensor], v_pages: Optional[torch.Tensor], nh: int,
+                    nkv: int, dim: int, vdim: int) -> torch.Tensor:
+    """From rows [q: nh dim | k: nkv dim | v: nkv vdim | ...]: biases, the norm over all of a row's queries (keys)
+    with weights wq (wk), the queries' factor 1 + temp_coef ln(floor((p + 1) / temp_every) + 1) (temp_every 0: none);
+    queries to ``q_out`` [N, nh dim], keys and values to their pages at ``slots`` (None: queries only)."""
+    N = proj.shape[0]
+    _rows(proj, nh * dim + (nkv * (dim + vdim) if slots is not None else 0), "sigattn_prepare rows")
+    _f32(bq, nh * dim, "sigattn_prepare bq"); _f32(bk, nkv * dim, "sigattn_prepare bk"); _f32(bv, nkv * vdim, "sigattn_prepare bv")
+    _f32(wq, nh * dim, "sigattn_prepare wq"); _f32(wk, nkv * dim, "sigattn_prepare wk")
+    _need(q_out.is_cuda and q_out.is_contiguous() and tuple(q_out.shape) == (N, nh * dim) and q_out.dtype == proj.dtype,
+          "sigattn_prepare: q_out [N, nh dim] of the rows' dtype")
+    _i32(positions, N, "sigattn_prepare positions")
+    ps = num_pages = 0
+    if slots is not None:
+        _i32(slots, N, "sigattn_prepare slots")
+        _dev(k_pages, v_pages)
+        num_pages, ps = k_pages.shape[0], k_pages.shape[2]
+        _need(tuple(k_pages.shape) == (num_pages, nkv, ps, dim) and tuple(v_pages.shape) == (num_pages, nkv, ps, vdim)
+              and k_pages.dtype == proj.dtype and v_pages.dtype == proj.dtype,
+              "sigattn_prepare: pages [P, nkv, page, dim] and [P, nkv, page, vdim] of the rows' dtype")
+    _ok(_core().ia_sigattn_prepare(_p(proj), DTYPE_CODE[proj.dtype], int(proj.stride(0)), _p(bq), _p(bk), _p(bv), _p(wq),
+                                   _p(wk), ctypes.c_float(eps), ctypes.c_float(temp_coef), int(temp_every),
+                                   _p(positions), _p(slots), _p(q_out), _p(k_pages), _p(v_pages), N, nh, nkv, dim, vdim,
+                                   ps, num_pages, _stream()), "sigattn_prepare")
+    return q_out
+
+
+def _check_sigattn(q, k_pages, v_pages, gate, out, nh, nkv, dim, vdim, what):
+    N = q.shape[0]
+    _rows(q, nh * dim, what + " queries")
+    _dev(k_pages, v_pages, out)
+    num_pages, ps = k_pages.shape[0], k_pages.shape[2]
+    _need(tuple(k_pages.shape) == (num_pages, nkv, ps, dim) and tuple(v_pages.shape) == (num_pages, nkv, ps, vdim)
+          and k_pages.dtype == q.dtype and v_pages.dtype == q.dtype, what + ": pages of the queries' dtype and sizes")
+    _need(tuple(out.shape) == (N, nh * vdim) and out.dtype == q.dtype, what + ": out [N, nh vdim]")
+    if gate is not None:
+        _rows(gate, nh, what + " gate")
+        _need(gate.dtype == q.dtype and gate.shape[0] == N, what + ": a gate row per query row")
+    return N, num_pages, ps
+
+
+def sigattn_generic(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, gate: Optional[torch.Tensor],
+                    out: torch.Tensor, token_seq: torch.Tensor, positions: torch.Tensor, block_tables: torch.Tensor,
+                    r1, r2, pb, nh: int, nkv: int, dim: int, vdim: int, scale: float) -> torch.Tensor:
+    """out[n, h] = sigmoid(gate[n, h]) sum_{j <= p} sigmoid(scale q.k_j - r1_h ln(1 + r2_h (p - j)) + pb_h) v_j, the
+    plain kernel (one wave per token and head, fp32 arithmetic)."""
+    N, num_pages, ps = _check_sigattn(q, k_pages, v_pages, gate, out, nh, nkv, dim, vdim, "sigattn_generic")
+    for t in (r1, r2, pb):
+        _f32(t, nh, "sigattn_generic per-head numbers")
+    _i32(token_seq, N, "sigattn token_seq"); _i32(positions, N, "sigattn positions")
+    _need(block_tables.dtype == torch.int32 and block_tables.dim() == 2 and block_tables.is_contiguous(), "sigattn: block tables")
+    _ok(_core().ia_sigattn_generic(_p(q), int(q.stride(0)), _p(k_pages), _p(v_pages), _p(gate),
+                                   int(gate.stride(0)) if gate is not None else 0, _p(out), DTYPE_CODE[q.dtype],
+                                   _p(token_seq), _p(positions), _p(block_tables), block_tables.shape[1], _p(r1), _p(r2),
+                                   _p(pb), N, nh, nkv, dim, vdim, ps, num_pages, ctypes.c_float(scale), _stream()),
+        "sigattn_generic")
+    return out
 
 
 # ------------------------------------------------------------------------- sampling

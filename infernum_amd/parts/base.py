@@ -33,7 +33,8 @@ class PartSpec:
 
 @dataclass(frozen=True)
 class WeightSpec:
-    """One tensor a part wants: its shape, how random weights are drawn for it,
+    """One tensor a part wants: its shape (a size of -1: whatever the file has; the part reads it off the tensor
+    when it loads, and random weights cannot be drawn for it), how random weights are drawn for it,
     whether it is a matrix that follows the compute dtype, and the full name of
     another tensor that stands in when the file does not hold this one."""
 

@@ -12,6 +12,13 @@ their matrix products) and the norm sits on each branch's output; the
 feed-forward (with its norm) may be absent.  One kernel normalises the branch,
 adds it into the fp32 stream and leaves the rounded stream for the next
 sublayer (``RMSNorm.add_normed``).
+
+``sandwich``: a norm before and after each sublayer, and optionally a gate on the sublayer's result that reads what
+the sublayer read:  a = norm1(h); h' = h + norm1b(gate1(a) * mixer(a));  f = norm2(h'); h'' = h' + norm2b(gate2(f) *
+feed_forward(f)).  The norms after the sublayers and the gates are extra parts (``mixer_post_norm``,
+``feed_forward_post_norm``: norms; ``mixer_gate``, ``feed_forward_gate``: category ``branch_gate``).  One kernel gates
+the branch, normalises it, adds it into the fp32 stream and, after the mixer, leaves the feed-forward's normalised
+input as well (``kernels.api.gated_norm_add``).
 """
 from __future__ import annotations
 
@@ -98,5 +105,76 @@ class BranchNormBlock(Block):
         program.x_holds_stream = program.h              # program.x is the stream, rounded, until a norm writes it
 
 
+class SandwichBlock(Block):
+    graph_safe = True
+
+    def __init__(self, rt, mixer, feed_forward, mixer_norm, feed_forward_norm, extra):
+        super().__init__(rt, mixer, feed_forward, mixer_norm, feed_forward_norm, extra)
+        from .rmsnorm import RMSNorm
+        for name in ("mixer_post_norm",) + (("feed_forward_post_norm",) if feed_forward is not None else ()):
+            if not isinstance(self.extra.get(name), RMSNorm):
+                raise ValueError(f"the sandwich arrangement needs an rmsnorm as {name!r}")
+        # the feed-forward's own norm rides on the kernel that adds the mixer's branch when it is the stock norm
+        self._fuse_next = (feed_forward is not None and type(feed_forward_norm) is RMSNorm
+                           and feed_forward_norm.eps == self.extra["mixer_post_norm"].eps)
+
+    def _branch(self, h, y, a, gate, post, next_norm=None):
+        from ..kernels import api as K
+        logits = gate.logits(a) if gate is not None else None
+        x = torch.empty_like(a) if next_norm is not None else None
+        K.gated_norm_add(h, y, logits, gate.bias if gate is not None else None, post.weight, post.eps,
+                         next_norm.weight if next_norm is not None else None, x)
+        return x
+
+    def forward(self, h: torch.Tensor, pending, ctx: StepContext, cache: CacheView):
+        a = self.mixer_norm.forward(h, pending)
+        y = self.mixer.forward(a, ctx, cache)
+        nxt = self.feed_forward_norm if self._fuse_next else None
+        f = self._branch(h, y, a, self.extra.get("mixer_gate"), self.extra["mixer_post_norm"], nxt)
+        if self.feed_forward is not None:
+            if f is None:
+                f = self.feed_forward_norm.forward(h, None)
+            y = self.feed_forward.forward(f, ctx)
+            self._branch(h, y, f, self.extra.get("feed_forward_gate"), self.extra["feed_forward_post_norm"])
+        return None
+
+    def _emit_branch(self, program, gate, post, key: str, next_norm=None) -> None:
+        """``program.x`` holds what the sublayer read, ``program.pending`` its result."""
+        from ..engine.program import STREAM
+        from ..kernels import api as K
+        H = program.hidden_size
+        logits = gate.emit_logits(program, key) if gate is not None else None
+        f32 = K.DTYPE_CODE[torch.float32]
+        program.keep(post.weight, next_norm.weight if next_norm is not None else None,
+                     gate.bias if gate is not None else None)
+        for alt in program.pending.alts:
+            if not alt.splits and alt.dtype != self.rt.dtype:
+                raise K.KernelError("gated_norm_add: the delta must have the activations' dtype")
+            code = f32 if alt.splits else program.act_code
+            program.op("core", "ia_gated_norm_add",
+                       [program.h, alt.where, code, alt.splits or 1, program.N, logits, f32, H,
+                        gate.bias if gate is not None else None, post.weight, K.DTYPE_CODE[post.weight.dtype],
+                        next_norm.weight if next_norm is not None else None,
+                        K.DTYPE_CODE[next_norm.weight.dtype] if next_norm is not None else 0,
+                        program.x if next_norm is not None else None, program.act_code, program.N, H, float(post.eps),
+                        STREAM], alt.when)
+        program.pending = None
+
+    def native(self, program, view: CacheView) -> None:
+        if type(self).forward is not SandwichBlock.forward:
+            return super().native(program, view)
+        self.mixer_norm.native(program, None)
+        self.mixer.native(program, view)
+        nxt = self.feed_forward_norm if self._fuse_next else None
+        self._emit_branch(program, self.extra.get("mixer_gate"), self.extra["mixer_post_norm"], "sandwich.gate1", nxt)
+        if self.feed_forward is not None:
+            if nxt is None:
+                self.feed_forward_norm.native(program, None)
+            self.feed_forward.native(program, None)
+            self._emit_branch(program, self.extra.get("feed_forward_gate"), self.extra["feed_forward_post_norm"],
+                              "sandwich.gate2")
+
+
 register_part("block", "prenorm", PreNormBlock)
 register_part("block", "branchnorm", BranchNormBlock)
+register_part("block", "sandwich", SandwichBlock)

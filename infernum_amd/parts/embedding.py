@@ -9,7 +9,7 @@ the two then share one buffer here.
 """
 from __future__ import annotations
 
-from typing import Dict, Optional
+from typing import Any, Dict, Mapping, Optional
 
 import torch
 
@@ -24,8 +24,9 @@ EMBEDDING_OUTPUT = "embedding.out"
 class TokenEmbedding(Embedding):
     graph_safe = True
     def __init__(self, rt: Runtime, vocab_size: int, hidden_size: int, init_std: float = 0.02, scale: float = 1.0,
-                 name: str = "weight", keep_output: bool = False):
-        """``scale`` multiplies the looked-up row in fp32 (the table itself stays as stored: a head tied to it
+                 name: str = "weight", keep_output: bool = False, position_table: Optional[Mapping[str, Any]] = None):
+        """``position_table`` {name, rows, init_std}: a learned vector per position, added (unscaled) to the token's row;
+        a position beyond its rows leaves NaN.  ``scale`` multiplies the looked-up row in fp32 (the table itself stays as stored: a head tied to it
         reads it unscaled); ``name`` is the table's local tensor name.  ``keep_output``: the rows as they leave
         here stay available to later parts of the step, rounded to the compute dtype (``EMBEDDING_OUTPUT`` in
         ``ctx.extras``, or the program's buffer of that name)."""
@@ -35,16 +36,26 @@ class TokenEmbedding(Embedding):
         self.init_std = init_std
         self.scale, self.name = float(scale), str(name)
         self.table: Optional[torch.Tensor] = None
+        self.position_table = dict(position_table) if position_table else None
+        self.pos_rows: Optional[torch.Tensor] = None
 
     def weights(self) -> Dict[str, WeightSpec]:
-        return {self.name: WeightSpec((self.vocab_size, self.hidden_size), ("normal", self.init_std))}
+        out = {self.name: WeightSpec((self.vocab_size, self.hidden_size), ("normal", self.init_std))}
+        if self.position_table:
+            out[self.position_table["name"]] = WeightSpec((int(self.position_table["rows"]), self.hidden_size),
+                                                          ("normal", self.position_table.get("init_std", self.init_std)))
+        return out
 
     def load(self, tensors: Dict[str, torch.Tensor]) -> None:
         self.table = tensors[self.name].contiguous()
+        if self.position_table:
+            self.pos_rows = tensors[self.position_table["name"]].contiguous()
 
     def forward(self, ctx: StepContext) -> torch.Tensor:
         h = torch.empty((ctx.num_tokens, self.hidden_size), dtype=torch.float32, device=self.table.device)
         K.embed(self.table, ctx.token_ids, h, self.scale)
+        if self.pos_rows is not None:
+            K.add_rows(h, self.pos_rows, ctx.positions)
         if self.keep_output:
             ctx.extras[EMBEDDING_OUTPUT] = K.cast(h, self.rt.dtype)
         return h
@@ -55,6 +66,10 @@ class TokenEmbedding(Embedding):
         from ..engine.program import STREAM
         program.op("core", "ia_embed", [self.table, K.DTYPE_CODE[self.table.dtype], program.token_ids, program.h,
                                         program.N, self.hidden_size, self.vocab_size, float(self.scale), STREAM])
+        if self.pos_rows is not None:
+            program.op("core", "ia_add_rows", [program.h, self.pos_rows, K.DTYPE_CODE[self.pos_rows.dtype],
+                                               program.positions, program.N, self.hidden_size,
+                                               int(self.pos_rows.shape[0]), STREAM])
         if self.keep_output:
             kept = program.buffer(EMBEDDING_OUTPUT, program.T * self.hidden_size * program.act_bytes)
             program.op("core", "ia_cast", [program.h, K.DTYPE_CODE[torch.float32], kept, program.act_code,
@@ -65,11 +80,13 @@ class TokenEmbedding(Embedding):
 class LinearHead(Head):
     graph_safe = True
     def __init__(self, rt: Runtime, vocab_size: int, hidden_size: int, fallback: Optional[str] = None,
-                 tied: bool = False, init_std: float = 0.02, name: str = "weight", softcap: Optional[float] = None):
-        """``softcap`` c: the logits become c tanh(logits / c).  ``name``: the matrix's local tensor name."""
+                 tied: bool = False, init_std: float = 0.02, name: str = "weight", softcap: Optional[float] = None,
+                 scale: float = 1.0):
+        """``scale`` s: the logits are multiplied by s (in fp32).  ``softcap`` c: the logits become c tanh(logits / c).  ``name``: the matrix's local tensor name."""
         super().__init__(rt)
         self.name = str(name)
         self.softcap = float(softcap) if softcap else 0.0
+        self.scale = float(scale)
         self.vocab_size, self.hidden_size = int(vocab_size), int(hidden_size)
         self.fallback, self.tied, self.init_std = fallback, bool(tied), init_std
         self.weight: Optional[torch.Tensor] = None
@@ -86,6 +103,8 @@ class LinearHead(Head):
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         logits = linear(x, self.weight, out_dtype=torch.float32, kernels=self.rt.kernels)
+        if self.scale != 1.0 and logits.shape[0]:
+            logits = K.scale_(logits if logits.is_contiguous() else logits.contiguous(), self.scale)
         if self.softcap and logits.shape[0]:
             logits = K.softcap(logits if logits.is_contiguous() else logits.contiguous(), self.softcap)
         return logits
@@ -94,8 +113,10 @@ class LinearHead(Head):
         if type(self).forward is not LinearHead.forward:
             return super().native(program, view)
         emit_linear(program, program.x, program.R, self.weight, torch.float32, None, False, program.logits, "head")
+        from ..engine.program import STREAM
+        if self.scale != 1.0:
+            program.op("core", "ia_scale", [program.logits, program.R, self.vocab_size, float(self.scale), STREAM])
         if self.softcap:
-            from ..engine.program import STREAM
             program.op("core", "ia_softcap", [program.logits, program.R, self.vocab_size, float(self.softcap), STREAM])
 
 

@@ -11,6 +11,13 @@ end in one thread of the product's tile) and [E, W, ff].  The tokens are grouped
 only the chosen experts' weights are read.  The result is left as fp32 parts [top, N, W], one per choice, each
 already times its weight, which the next norm adds in the order of the choices: an expert's output is never
 rounded to the compute dtype.
+
+Options for other designs.  ``gated=False``: an expert is D_e act(U_e x) without a gate (``activation`` names the
+function: ``relu_squared``, ``gelu``, ``gelu_tanh``; tensors ``e<i>.up`` and ``e<i>.down``).  ``router="softmax_top"``:
+s = softmax(z) over ALL experts, the ``top`` largest of s + correction are chosen (``correction``: a stored vector that
+moves the choice only), and the weights are the chosen s over their sum (+ 1e-20).  ``shared_ff``: one more expert of
+that middle width (``shared.up``, ``shared.down``; same form, no gate) that every token takes with weight 1; its
+result is added into the first choice's part.
 """
 from __future__ import annotations
 
@@ -27,16 +34,27 @@ class RoutedExperts(FeedForward):
     graph_safe = True
 
     def __init__(self, rt: Runtime, hidden_size: int, intermediate_size: int, num_experts: int, top: int,
-                 limit: float, alpha: float = 1.702, router_bias: bool = True, router_name: str = "router",
-                 expert_prefix: str = "e", init_std: float = 0.02):
+                 limit: Optional[float] = None, alpha: float = 1.702, router_bias: bool = True,
+                 router_name: str = "router", expert_prefix: str = "e", init_std: float = 0.02, gated: bool = True,
+                 activation: str = "relu_squared", router: str = "top_softmax", correction_name: str = "correction",
+                 shared_ff: Optional[int] = None):
         super().__init__(rt)
         self.hidden_size, self.ff = int(hidden_size), int(intermediate_size)
         self.num_experts, self.top = int(num_experts), int(top)
         if not 0 < self.top <= self.num_experts:
             raise ValueError(f"a token takes {top} of {num_experts} experts")
-        self.limit, self.alpha = float(limit), float(alpha)
-        if not self.limit > 0:
+        self.gated, self.activation, self.router = bool(gated), str(activation), str(router)
+        if self.router not in ("top_softmax", "softmax_top"):
+            raise ValueError(f"router {router!r}: 'top_softmax' or 'softmax_top'")
+        if not self.gated and self.activation not in K.ACTIVATIONS:
+            raise ValueError(f"activation {activation!r}: one of {sorted(K.ACTIVATIONS)}")
+        self.limit, self.alpha = float(limit) if limit is not None else 0.0, float(alpha)
+        if self.gated and not self.limit > 0:
             raise ValueError("the experts' limit must be positive")
+        self.correction_name = correction_name
+        self.shared_ff = int(shared_ff) if shared_ff else 0
+        if self.shared_ff and self.gated:
+            raise ValueError("a shared expert goes with experts without a gate")
         self.router_bias, self.router_name, self.expert_prefix = bool(router_bias), router_name, expert_prefix
         self.init_std = init_std
         self.w_router: Optional[torch.Tensor] = None
@@ -48,11 +66,17 @@ class RoutedExperts(FeedForward):
         H, I, E = self.hidden_size, self.ff, self.num_experts
         init = ("normal", self.init_std)
         out = {self.router_name: WeightSpec((E, H), init)}
-        if self.router_bias:
+        if self.router == "softmax_top":
+            out[self.correction_name] = WeightSpec((E,), ("normal", 0.05), follows_compute_dtype=False)
+        elif self.router_bias:
             out[self.router_name + ".b"] = WeightSpec((E,), ("normal", 0.5), follows_compute_dtype=False)
+        if self.shared_ff:
+            out["shared.up"] = WeightSpec((self.shared_ff, H), init)
+            out["shared.down"] = WeightSpec((H, self.shared_ff), init)
         for e in range(E):
             p = f"{self.expert_prefix}{e}."
-            out[p + "gate"] = WeightSpec((I, H), init)
+            if self.gated:
+                out[p + "gate"] = WeightSpec((I, H), init)
             out[p + "up"] = WeightSpec((I, H), init)
             out[p + "down"] = WeightSpec((H, I), init)
         return out
@@ -60,23 +84,40 @@ class RoutedExperts(FeedForward):
     def load(self, tensors: Dict[str, torch.Tensor]) -> None:
         H, I, E = self.hidden_size, self.ff, self.num_experts
         self.w_router = tensors[self.router_name].contiguous()
-        self.b_router = tensors[self.router_name + ".b"].contiguous() if self.router_bias else None
+        if self.router == "softmax_top":
+            self.b_router = tensors[self.correction_name].contiguous()
+        else:
+            self.b_router = tensors[self.router_name + ".b"].contiguous() if self.router_bias else None
         dev, dt = self.w_router.device, self.w_router.dtype
-        self.w_gate_up = torch.empty((E, 2 * I, H), dtype=dt, device=dev)
+        self.w_gate_up = torch.empty((E, (2 if self.gated else 1) * I, H), dtype=dt, device=dev)
         self.w_down = torch.empty((E, H, I), dtype=dt, device=dev)
         for e in range(E):
             p = f"{self.expert_prefix}{e}."
-            self.w_gate_up[e, 0::2] = tensors[p + "gate"]
-            self.w_gate_up[e, 1::2] = tensors[p + "up"]
+            if self.gated:
+                self.w_gate_up[e, 0::2] = tensors[p + "gate"]
+                self.w_gate_up[e, 1::2] = tensors[p + "up"]
+            else:
+                self.w_gate_up[e] = tensors[p + "up"]
             self.w_down[e] = tensors[p + "down"]
+        if self.shared_ff:
+            from .linear import prepare_weights
+            self.w_shared_up, self.w_shared_down = tensors["shared.up"].contiguous(), tensors["shared.down"].contiguous()
+            prepare_weights(self.rt, [(self.w_shared_up, None, False), (self.w_shared_down, None, False)])
 
     def forward(self, x: torch.Tensor, ctx: Optional[StepContext] = None):
         z = linear(x, self.w_router, out_dtype=torch.float32, kernels=self.rt.kernels)
-        ids, weights = K.router_topk(z, self.b_router, self.top)
-        return K.moe_experts(x, ids, weights, self.w_gate_up, self.w_down, self.limit, self.alpha)
+        choose = K.router_softmax_topk if self.router == "softmax_top" else K.router_topk
+        ids, weights = choose(z, self.b_router, self.top)
+        if self.gated:
+            return K.moe_experts(x, ids, weights, self.w_gate_up, self.w_down, self.limit, self.alpha)
+        parts = K.moe_plain_experts(x, ids, weights, self.w_gate_up, self.w_down, self.activation)
+        if self.shared_ff:
+            u = K.activation(linear(x, self.w_shared_up, kernels=self.rt.kernels), self.activation)
+            K.stream_add(parts[0], linear(u, self.w_shared_down, out_dtype=torch.float32, kernels=self.rt.kernels))
+        return K.SplitSum(parts)
 
     def native(self, program, view=None) -> None:
-        if type(self).forward is not RoutedExperts.forward:
+        if type(self).forward is not RoutedExperts.forward or not self.gated or self.router != "top_softmax":
             return super().native(program, view)
         from ..engine.program import ALWAYS, STREAM, Alt, Value
         H, I, E, top, T, N = self.hidden_size, self.ff, self.num_experts, self.top, program.T, program.N

@@ -1,0 +1,108 @@
+"""Attention over the paged cache whose weights are sigmoids, not a softmax.
+
+q = x Wq^T + bq, k = x Wk^T + bk (heads of ``head_dim``), v = x Wv^T + bv (heads of ``value_dim``); all of a token's
+queries together are divided by their root mean square and multiplied by a weight per value, and so are all of its
+keys; the queries are multiplied by 1 + coef ln(floor((p + 1) / every) + 1) at position p when the mixer has such a
+factor.  There is no rotation.  Query head h reads key/value head h // (nh / nkv); for the key at j <= p
+
+    w = sigmoid( scale q.k_j - r1_h ln(1 + r2_h (p - j)) + b_h ),     out_h = sigmoid(gate_h) sum_j w v_j,
+
+with nothing normalised over the keys, r1, r2, b numbers per head and gate = x Wg^T one number per token and head.
+Then the output projection.  One product makes q, k, v and the gates' logits; keys are kept [nkv, page, head_dim]
+and values [nkv, page, value_dim] per page.  Scores, the distance term, sigmoids and the sums over the keys are fp32.
+"""
+from __future__ import annotations
+
+from typing import Any, Dict, Mapping, Optional
+
+import torch
+
+from ..kernels import api as K
+from .base import CacheSpec, CacheView, Mixer, PageTensor, Runtime, StepContext, WeightSpec, register_part
+from .linear import emit_linear, linear, prepare_weights
+
+
+class SigmoidAttention(Mixer):
+    graph_safe = True
+
+    def __init__(self, rt: Runtime, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int, value_dim: int,
+                 scale: float, norm_eps: float, q_temp: Optional[Mapping[str, Any]] = None, biases: bool = True,
+                 gate: bool = True, distance_bias: bool = True, init_std: float = 0.02):
+        """``q_temp`` {coef, every} or None; ``biases``: q, k and v have them; ``gate``: a sigmoid gate per token and
+        head on the output; ``distance_bias``: the heads have r1, r2 (the term r1 ln(1 + r2 distance) taken off the
+        score) and the number b added to it."""
+        super().__init__(rt)
+        if num_heads % num_kv_heads:
+            raise ValueError(f"num_heads {num_heads} is not a multiple of num_kv_heads {num_kv_heads}")
+        self.hidden_size, self.nh, self.nkv = int(hidden_size), int(num_heads), int(num_kv_heads)
+        self.dim, self.vdim = int(head_dim), int(value_dim)
+        if max(self.dim, self.vdim) > K.GENERIC_MAX_HEAD_DIM:
+            raise ValueError(f"head sizes above {K.GENERIC_MAX_HEAD_DIM} have no attention kernel")
+        self.scale, self.norm_eps = float(scale), float(norm_eps)
+        self.temp_coef = float(q_temp["coef"]) if q_temp else 0.0
+        self.temp_every = int(q_temp["every"]) if q_temp else 0
+        self.biases, self.gate, self.distance_bias, self.init_std = bool(biases), bool(gate), bool(distance_bias), init_std
+        self.nq, self.nk, self.nv = self.nh * self.dim, self.nkv * self.dim, self.nkv * self.vdim
+        self.row = self.nq + self.nk + self.nv + (self.nh if self.gate else 0)
+        self.bq = self.bk = self.bv = self.r1 = self.r2 = self.pb = None
+
+    # ---- what it needs ---------------------------------------------------
+    def cache_spec(self) -> CacheSpec:
+        return CacheSpec("full", payload=(PageTensor("k", (self.nkv, self.dim), token_axis=1),
+                                          PageTensor("v", (self.nkv, self.vdim), token_axis=1)))
+
+    def weights(self) -> Dict[str, WeightSpec]:
+        H, init, small = self.hidden_size, ("normal", self.init_std), dict(follows_compute_dtype=False)
+        out = {"q": WeightSpec((self.nq, H), init), "k": WeightSpec((self.nk, H), init), "v": WeightSpec((self.nv, H), init),
+               "q.norm": WeightSpec((self.nq,), ("uniform", 0.8, 1.2), **small),
+               "k.norm": WeightSpec((self.nk,), ("uniform", 0.8, 1.2), **small),
+               "o": WeightSpec((H, self.nh * self.vdim), init)}
+        if self.biases:
+            out.update({"q.b": WeightSpec((self.nq,), ("normal", 0.1), **small),
+                        "k.b": WeightSpec((self.nk,), ("normal", 0.1), **small),
+                        "v.b": WeightSpec((self.nv,), ("normal", 0.1), **small)})
+        if self.distance_bias:
+            out.update({"r1": WeightSpec((self.nh,), ("uniform", 0.2, 1.0), **small),
+                        "r2": WeightSpec((self.nh,), ("uniform", 0.05, 0.5), **small),
+                        "pb": WeightSpec((self.nh,), ("uniform", -3.0, -1.0), **small)})
+        if self.gate:
+            out["g"] = WeightSpec((self.nh, H), init)
+        return out
+
+    def load(self, tensors: Dict[str, torch.Tensor]) -> None:
+        f32 = lambda name: tensors[name].to(torch.float32).contiguous()           # noqa: E731
+        rows = [tensors["q"], tensors["k"], tensors["v"]] + ([tensors["g"]] if self.gate else [])
+        self.w_in = torch.cat(rows, dim=0).contiguous()
+        self.w_o = tensors["o"].contiguous()
+        self.wq, self.wk = f32("q.norm"), f32("k.norm")
+        if self.biases:
+            self.bq, self.bk, self.bv = f32("q.b"), f32("k.b"), f32("v.b")
+        if self.distance_bias:
+            self.r1, self.r2, self.pb = f32("r1"), f32("r2"), f32("pb")
+        prepare_weights(self.rt, [(self.w_in, None, False), (self.w_in[: self.nq], None, False), (self.w_o, None, True)])
+
+    # ---- one step --------------------------------------------------------
+    def forward(self, x: torch.Tensor, ctx: StepContext, cache: CacheView):
+        if cache.k_pages is None or cache.v_pages is None:
+            raise K.KernelError("attention needs pages of the cache")
+        if not cache.writable:
+            raise K.KernelError("sigmoid_attention: every run writes its own keys and values")
+        n, g = x.shape[0], cache.group
+        proj = linear(x, self.w_in, kernels=self.rt.kernels)                     # [n, q | k | v | gate logits]
+        q = torch.empty((n, self.nq), dtype=self.rt.dtype, device=x.device)
+        K.sigattn_prepare(proj, self.bq, self.bk, self.bv, self.wq, self.wk, self.norm_eps, self.temp_coef,
+                          self.temp_every, ctx.positions, ctx.slots[g], q, cache.k_pages, cache.v_pages, self.nh,
+                          self.nkv, self.dim, self.vdim)
+        out = torch.empty((n, self.nh * self.vdim), dtype=self.rt.dtype, device=x.device)
+        gate = proj[:, self.nq + self.nk + self.nv:] if self.gate else None
+        self.attend(q, gate, out, ctx, cache)
+        return linear(out, self.w_o, keep_split=True, kernels=self.rt.kernels)
+
+    def attend(self, q: torch.Tensor, gate: Optional[torch.Tensor], out: torch.Tensor, ctx: StepContext,
+               cache: CacheView) -> None:
+        K.sigattn_generic(q, cache.k_pages, cache.v_pages, gate, out, ctx.token_seq, ctx.positions,
+                          ctx.block_tables[cache.group], self.r1, self.r2, self.pb, self.nh, self.nkv, self.dim, self.vdim,
+                          self.scale)
+
+
+register_part("mixer", "sigmoid_attention", SigmoidAttention)

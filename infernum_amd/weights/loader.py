@@ -56,6 +56,11 @@ def _convert(t: torch.Tensor, spec: WeightSpec, rt: Runtime) -> torch.Tensor:
     return t.to(target).contiguous()                # float16 and float64 files, and hosts without a GPU
 
 
+def _shape_fits(found: tuple, wanted: tuple) -> bool:
+    """A wanted size of -1 is taken from the file (a part that reads a size off its tensors)."""
+    return len(found) == len(wanted) and all(w == -1 or int(f) == int(w) for f, w in zip(found, wanted))
+
+
 def check_against(expected: Dict[str, WeightSpec], found: Dict[str, tuple], where: str) -> Dict[str, str]:
     """Compare names and shapes; returns expected name -> name to read it from."""
     missing, wrong = [], []
@@ -69,7 +74,7 @@ def check_against(expected: Dict[str, WeightSpec], found: Dict[str, tuple], wher
             missing.append(name)
             continue
         used.add(src)
-        if tuple(found[src]) != tuple(spec.shape):
+        if not _shape_fits(found[src], spec.shape):
             wrong.append(f"{name}: expected {list(spec.shape)} got {list(found[src])}")
         source[name] = src
     unexpected = sorted(n for n in found if n not in used and n not in expected
