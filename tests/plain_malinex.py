@@ -134,18 +134,23 @@ def small_ff(f: torch.Tensor, up: torch.Tensor, down: torch.Tensor, act: Callabl
     return _r(act(_r(f @ up.T, round_to)), round_to) @ down.T
 
 
-def router(f: torch.Tensor, wr: torch.Tensor, correction: torch.Tensor, top: int):
+def router(f: torch.Tensor, wr: torch.Tensor, correction: torch.Tensor, top: int, margins: Optional[List] = None):
     """-> (chosen [T, top], weights [T, top]): softmax over all experts; the choice goes by score + correction, the
-    weights are the chosen scores themselves over their sum."""
+    weights are the chosen scores themselves over their sum.  ``margins`` collects, per token, by how much the last
+    chosen expert beats the first that is not, as a fraction of the largest choice score."""
     s = torch.softmax(f @ wr.T, dim=-1)
+    c = torch.sort(s + correction, dim=-1, descending=True).values
+    if margins is not None and top < c.shape[1]:
+        margins.append((c[:, top - 1] - c[:, top]) / c[:, 0].abs().clamp_min(1e-30))
     chosen = torch.topk(s + correction, top, dim=-1).indices
     picked = torch.gather(s, 1, chosen)
     return chosen, picked / (picked.sum(dim=-1, keepdim=True) + 1e-20)
 
 
-def routed_ff(f: torch.Tensor, w: Mapping[str, torch.Tensor], p: str, mlp: Mapping, round_to=None) -> torch.Tensor:
+def routed_ff(f: torch.Tensor, w: Mapping[str, torch.Tensor], p: str, mlp: Mapping, round_to=None,
+              margins: Optional[List] = None) -> torch.Tensor:
     E, top = mlp["router"]["experts"], mlp["router"]["top"]
-    chosen, weights = router(f, w[p + "router"], w[p + "correction"], top)
+    chosen, weights = router(f, w[p + "router"], w[p + "correction"], top, margins)
     out = torch.zeros((f.shape[0], w[p + "e0.down"].shape[0]), dtype=F64)
     for t in range(f.shape[0]):
         for c in range(top):
@@ -156,36 +161,117 @@ def routed_ff(f: torch.Tensor, w: Mapping[str, torch.Tensor], p: str, mlp: Mappi
     return out
 
 
-def feed_forward(f: torch.Tensor, w: Mapping[str, torch.Tensor], p: str, mlp: Mapping, round_to=None) -> torch.Tensor:
+def feed_forward(f: torch.Tensor, w: Mapping[str, torch.Tensor], p: str, mlp: Mapping, round_to=None,
+                 margins: Optional[List] = None) -> torch.Tensor:
     if mlp["kind"] == "dense":
         return _r(small_ff(f, w[p + "up"], w[p + "down"], gelu_erf, round_to), round_to)
-    return routed_ff(f, w, p, mlp, round_to)
+    return routed_ff(f, w, p, mlp, round_to, margins)
 
 
 # --------------------------------------------------------------------------------------------- the model
-def layer(x: torch.Tensor, w: Mapping[str, torch.Tensor], p: str, entry: Mapping, eps: float, round_to=None) -> torch.Tensor:
+def layer(x: torch.Tensor, w: Mapping[str, torch.Tensor], p: str, entry: Mapping, eps: float, round_to=None,
+          margins: Optional[List] = None) -> torch.Tensor:
     a = _r(rms_norm(x, w[p + "norm1"], eps), round_to)
     mix = gla_mixer if entry["type"] == "gla" else attention_mixer
     y = mix(a, w, p + "mix.", entry["mixer"], eps, round_to) * sigmoid(a @ w[p + "rg1"].T + w[p + "rg1.b"])
     x = x + rms_norm(y, w[p + "norm1b"], eps)
     if entry.get("mlp") is not None:
         f = _r(rms_norm(x, w[p + "norm2"], eps), round_to)
-        y = feed_forward(f, w, p + "mlp.", entry["mlp"], round_to) * sigmoid(f @ w[p + "rg2"].T + w[p + "rg2.b"])
+        y = feed_forward(f, w, p + "mlp.", entry["mlp"], round_to, margins) * sigmoid(f @ w[p + "rg2"].T + w[p + "rg2.b"])
         x = x + rms_norm(y, w[p + "norm2b"], eps)
     return x
 
 
 def forward(config: Mapping, weights: Mapping[str, torch.Tensor], tokens, round_to=None,
-            streams: Optional[List[torch.Tensor]] = None, layers: Optional[int] = None) -> torch.Tensor:
+            streams: Optional[List[torch.Tensor]] = None, layers: Optional[int] = None,
+            margins: Optional[List] = None) -> torch.Tensor:
     """Logits [T, vocab] of one sequence from its first token.  ``streams`` collects the stream after every layer;
-    ``layers`` stops after so many."""
+    ``layers`` stops after so many; ``margins`` collects the routers' margins (see ``router``)."""
     w = {k: v.to(F64) for k, v in weights.items()}
     tokens = torch.as_tensor(tokens, dtype=torch.long)
     eps = float(config["norm"]["eps"])
     x = embed(tokens, w["embed"], torch.arange(tokens.numel()), w["pos"])
     for i, entry in enumerate(config["layers"][:layers]):
-        x = layer(x, w, f"l{entry.get('weights_of', i)}.", entry, eps, round_to)
+        x = layer(x, w, f"l{entry.get('weights_of', i)}.", entry, eps, round_to, margins)
         if streams is not None:
             streams.append(x.clone())
     x = _r(rms_norm(x, w["final.norm"], eps), round_to)
     return (x @ w["head"].T) * float(config.get("logit_scale", 1.0))
+
+
+# ------------------------------------------------------------------------------------------- test models
+def tensor_shapes(cfg: Mapping) -> Dict[str, tuple]:
+    """Name -> shape of every tensor a file of this configuration holds (a gla mixer's ``rank`` is the width of its
+    decay logits' middle)."""
+    W, out = cfg["width"], {}
+    out["embed"], out["pos"] = (cfg["vocab"], W), (cfg["max_positions"], W)
+    for i, entry in enumerate(cfg["layers"]):
+        if "weights_of" in entry:
+            continue
+        p, m = f"l{i}.", entry["mixer"]
+        for n in ("norm1", "norm1b"):
+            out[p + n] = (W,)
+        out[p + "rg1"], out[p + "rg1.b"] = (W, W), (W,)
+        if entry["type"] == "gla":
+            nq, nv = m["heads"] * m["dim"], m["heads"] * m["vdim"]
+            out.update({p + "mix.q": (nq, W), p + "mix.k": (nq, W), p + "mix.v": (nv, W), p + "mix.g": (nv, W),
+                        p + "mix.o": (W, nv), p + "mix.norm": (m["vdim"],), p + "mix.a1": (m["rank"], W),
+                        p + "mix.a2": (nq, m["rank"]), p + "mix.a2.b": (nq,)})
+        else:
+            H, G = m["heads"], m.get("kv_heads", m["heads"])
+            nq, nk, nv = H * m["dim"], G * m["dim"], G * m["vdim"]
+            out.update({p + "mix.q": (nq, W), p + "mix.q.b": (nq,), p + "mix.k": (nk, W), p + "mix.k.b": (nk,),
+                        p + "mix.v": (nv, W), p + "mix.v.b": (nv,), p + "mix.q.norm": (nq,), p + "mix.k.norm": (nk,),
+                        p + "mix.r1": (H,), p + "mix.r2": (H,), p + "mix.pb": (H,), p + "mix.g": (H, W),
+                        p + "mix.o": (W, H * m["vdim"])})
+        mlp = entry.get("mlp")
+        if mlp is None:
+            continue
+        for n in ("norm2", "norm2b"):
+            out[p + n] = (W,)
+        out[p + "rg2"], out[p + "rg2.b"] = (W, W), (W,)
+        if mlp["kind"] == "dense":
+            out[p + "mlp.up"], out[p + "mlp.down"] = (mlp["ff"], W), (W, mlp["ff"])
+        else:
+            E, ff = mlp["router"]["experts"], mlp["expert"]["ff"]
+            for e in range(E):
+                out[p + f"mlp.e{e}.up"], out[p + f"mlp.e{e}.down"] = (ff, W), (W, ff)
+            out[p + "mlp.router"], out[p + "mlp.correction"] = (E, W), (E,)
+            if mlp.get("shared") is not None:
+                sf = mlp["shared"]["ff"]
+                out[p + "mlp.shared.up"], out[p + "mlp.shared.down"] = (sf, W), (W, sf)
+    out["final.norm"], out["head"] = (W,), (cfg["vocab"], W)
+    return out
+
+
+def random_weights(cfg: Mapping, seed: int = 0, store: torch.dtype = torch.bfloat16) -> Dict[str, torch.Tensor]:
+    """Weights of a size that keeps every branch of order one; rounded to ``store``."""
+    g = torch.Generator().manual_seed(seed)
+    out = {}
+    for name, shape in tensor_shapes(cfg).items():
+        last = name.rsplit(".", 1)[-1]
+        rnd = lambda: torch.randn(shape, generator=g)                               # noqa: E731
+        if "norm" in last:
+            t = 1.0 + 0.2 * rnd()
+        elif name.endswith("a2.b"):
+            t = 1.0 + 3.0 * torch.rand(shape, generator=g)           # decays between forgetting fast and slowly
+        elif last == "b":
+            t = 0.5 * rnd()
+        elif last == "r1":
+            t = 0.2 + 0.8 * torch.rand(shape, generator=g)
+        elif last == "r2":
+            t = 0.05 + 0.5 * torch.rand(shape, generator=g)
+        elif last == "pb":
+            t = -3.0 + 2.0 * torch.rand(shape, generator=g)
+        elif last == "correction":
+            t = 0.05 * rnd()
+        elif name == "embed":
+            t = rnd()
+        elif name == "pos":
+            t = 0.5 * rnd()
+        elif last == "router":
+            t = 3.0 * rnd() / math.sqrt(shape[-1])
+        else:
+            t = rnd() / math.sqrt(shape[-1])
+        out[name] = t.to(store)
+    return out
