@@ -91,5 +91,26 @@ class GatedLinearAttention(Mixer):
         K.head_norm_gate(o, proj, self.g_col, self.w_norm, self.norm_eps, self.nh, self.vdim, gated)
         return linear(gated, self.w_o, keep_split=True, kernels=self.rt.kernels)
 
+    def native(self, program, view: CacheView) -> None:
+        if type(self).forward is not GatedLinearAttention.forward:
+            return super().native(program, view)
+        from ..engine.program import STREAM
+        rt, N, T, act, ab = self.rt, program.N, program.T, program.act_code, program.act_bytes
+        nq, nv = self.nh * self.dim, self.nh * self.vdim
+        state = self._state(view)
+        program.keep(state, self.b_a2, self.w_norm)
+        proj = emit_linear(program, program.x, N, self.w_in, rt.dtype, None, False, "gla.proj", "gla.in").tensor()
+        mid = emit_linear(program, program.x, N, self.w_a1, rt.dtype, None, False, "gla.mid", "gla.a1").tensor()
+        z = emit_linear(program, mid, N, self.w_a2, torch.float32, None, False, "gla.z", "gla.a2").tensor()
+        o = program.buffer("gla.o", T * nv * 4)
+        program.op("core", "ia_gla_scan", [proj, act, self.row, self.q_col, self.k_col, self.v_col, z, nq, self.b_a2,
+                                           float(self.tau), float(self.q_scale), state, int(state.stride(0)), o,
+                                           program.seq_starts, program.state_slots, program.B, self.nh, self.dim,
+                                           self.vdim, STREAM])
+        gated = program.buffer("gla.gated", T * nv * ab)
+        program.op("core", "ia_head_norm_gate", [o, proj, act, self.row, self.g_col, self.w_norm, gated, N, self.nh,
+                                                 self.vdim, float(self.norm_eps), STREAM])
+        program.pending = emit_linear(program, gated, N, self.w_o, rt.dtype, None, True, "gla.out", "gla.o_proj")
+
 
 register_part("mixer", "gla", GatedLinearAttention)

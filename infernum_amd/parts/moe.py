@@ -117,7 +117,7 @@ class RoutedExperts(FeedForward):
         return K.SplitSum(parts)
 
     def native(self, program, view=None) -> None:
-        if type(self).forward is not RoutedExperts.forward or not self.gated or self.router != "top_softmax":
+        if type(self).forward is not RoutedExperts.forward:
             return super().native(program, view)
         from ..engine.program import ALWAYS, STREAM, Alt, Value
         H, I, E, top, T, N = self.hidden_size, self.ff, self.num_experts, self.top, program.T, program.N
@@ -130,9 +130,12 @@ class RoutedExperts(FeedForward):
         y = program.buffer("moe.y", T * top * I * program.act_bytes)
         parts = program.buffer("moe.parts", top * T * H * 4)
         b = self.b_router
-        program.op("core", "ia_router_topk", [z.tensor(), b, K.DTYPE_CODE[b.dtype] if b is not None else 0, ids, wts,
-                                              N, E, top, STREAM])
+        choose = "ia_router_softmax_topk" if self.router == "softmax_top" else "ia_router_topk"
+        program.op("core", choose, [z.tensor(), b, K.DTYPE_CODE[b.dtype] if b is not None else 0, ids, wts,
+                                    N, E, top, STREAM])
         program.op("core", "ia_moe_sort", [ids, offsets, perm, N * top, E, STREAM])
+        if not self.gated:
+            return self._native_plain(program, ids, wts, offsets, perm, y, parts)
         from ..engine.program import NEVER, Guard
         first = K.moe_grouped_from_tokens(E, top, H, I, self.rt.dtype)
         grouped = Guard.between(N, first) if first > 0 else NEVER
@@ -151,6 +154,38 @@ class RoutedExperts(FeedForward):
             program.op("core", "ia_moe_glu", [gu, y, N * top, I, self.limit, self.alpha, STREAM], grouped)
             program.op("core", "ia_gemm_mfma_grouped", [y, self.w_down, xs, offsets, E, N * top, H, I, STREAM], grouped)
             program.op("core", "ia_moe_scatter", [xs, perm, wts, parts, N, top, H, STREAM], grouped)
+        program.pending = Value(H, [Alt(ALWAYS, parts, top, torch.float32)])
+
+
+    def _native_plain(self, program, ids, wts, offsets, perm, y, parts) -> None:
+        """The launches of ``kernels.api.moe_plain_experts`` and of the shared expert."""
+        from ..engine.program import ALWAYS, NEVER, STREAM, Alt, Guard, Value
+        from .linear import emit_linear as emit
+        H, I, E, top, T, N = self.hidden_size, self.ff, self.num_experts, self.top, program.T, program.N
+        act, code = K.ACTIVATIONS[self.activation], program.act_code
+        first = K.moe_grouped_from_tokens(E, top, H, I, self.rt.dtype)
+        grouped = Guard.between(N, first) if 0 < first <= T else NEVER
+        tiled = ~grouped
+        program.op("core", "ia_moe_up", [program.x, self.w_gate_up, y, offsets, perm, code, N * top, E, top, H, I, act,
+                                         STREAM], tiled)
+        program.op("core", "ia_moe_down", [y, self.w_down, parts, wts, offsets, perm, code, N, E, top, H, I, STREAM],
+                   tiled)
+        if 0 < first <= T:
+            xs = program.buffer("moe.sorted", T * top * H * program.act_bytes)
+            program.op("core", "ia_moe_gather", [program.x, perm, xs, N * top, top, H, STREAM], grouped)
+            program.op("core", "ia_gemm_mfma_grouped", [xs, self.w_gate_up, y, offsets, E, N * top, I, H, STREAM], grouped)
+            program.op("core", "ia_activation", [y, y, code, N * (top * I), act, STREAM], grouped)
+            program.op("core", "ia_gemm_mfma_grouped", [y, self.w_down, xs, offsets, E, N * top, H, I, STREAM], grouped)
+            program.op("core", "ia_moe_scatter", [xs, perm, wts, parts, N, top, H, STREAM], grouped)
+        if self.shared_ff:
+            program.keep(self.w_shared_up, self.w_shared_down)
+            u = emit(program, program.x, N, self.w_shared_up, self.rt.dtype, None, False, "moe.shared.act",
+                     "moe.shared.up").tensor()
+            program.op("core", "ia_activation", [u, u, code, N * self.shared_ff, act, STREAM])
+            down = emit(program, u, N, self.w_shared_down, torch.float32, None, True, "moe.shared.out", "moe.shared.down")
+            f32 = K.DTYPE_CODE[torch.float32]
+            for alt in down.alts:
+                program.op("core", "ia_stream_add", [parts, alt.where, f32, alt.splits or 1, N, H, STREAM], alt.when)
         program.pending = Value(H, [Alt(ALWAYS, parts, top, torch.float32)])
 
 

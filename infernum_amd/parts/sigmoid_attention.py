@@ -98,6 +98,36 @@ class SigmoidAttention(Mixer):
         self.attend(q, gate, out, ctx, cache)
         return linear(out, self.w_o, keep_split=True, kernels=self.rt.kernels)
 
+    def native(self, program, view: CacheView) -> None:
+        if type(self).forward is not SigmoidAttention.forward or type(self).attend is not SigmoidAttention.attend:
+            return super().native(program, view)
+        from ..engine.program import STREAM
+        if view.k_pages is None or view.v_pages is None or not view.writable:
+            raise K.KernelError("sigmoid_attention: every run needs pages of its own")
+        rt, N, T, act, ab = self.rt, program.N, program.T, program.act_code, program.act_bytes
+        k, v, g = view.k_pages, view.v_pages, view.group
+        ps, num_pages = int(k.shape[2]), int(k.shape[0])
+        program.keep(k, v, self.bq, self.bk, self.bv, self.wq, self.wk, self.r1, self.r2, self.pb)
+        proj = emit_linear(program, program.x, N, self.w_in, rt.dtype, None, False, "sigattn.proj", "sigattn.in").tensor()
+        q = program.buffer("sigattn.q", T * self.nq * ab)
+        program.op("core", "ia_sigattn_prepare", [proj, act, self.row, self.bq, self.bk, self.bv, self.wq, self.wk,
+                                                  float(self.norm_eps), float(self.temp_coef), int(self.temp_every),
+                                                  program.positions, program.slots(g), q, k, v, N, self.nh, self.nkv,
+                                                  self.dim, self.vdim, ps, num_pages, STREAM])
+        out = program.buffer("sigattn.out", T * self.nh * self.vdim * ab)
+        gate = proj.at((self.nq + self.nk + self.nv) * ab) if self.gate else None
+        self.emit_attend(program, view, q, gate, out)
+        program.pending = emit_linear(program, out, N, self.w_o, rt.dtype, None, True, "sigattn.o", "sigattn.o_proj")
+
+    def emit_attend(self, program, view: CacheView, q, gate, out) -> None:
+        from ..engine.program import STREAM
+        k, v, g = view.k_pages, view.v_pages, view.group
+        program.op("core", "ia_sigattn_generic", [q, self.nq, k, v, gate, self.row if gate is not None else 0, out,
+                                                  program.act_code, program.token_seq, program.positions,
+                                                  program.block_table(g), program.bt_cols(g), self.r1, self.r2, self.pb,
+                                                  program.N, self.nh, self.nkv, self.dim, self.vdim, int(k.shape[2]),
+                                                  int(k.shape[0]), float(self.scale), STREAM])
+
     def attend(self, q: torch.Tensor, gate: Optional[torch.Tensor], out: torch.Tensor, ctx: StepContext,
                cache: CacheView) -> None:
         K.sigattn_generic(q, cache.k_pages, cache.v_pages, gate, out, ctx.token_seq, ctx.positions,

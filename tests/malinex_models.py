@@ -11,7 +11,7 @@ X2: sizes that no fast kernel takes (width 100, odd vocabulary, heads of 26 and 
 X3: twenty heads over one key/value head, keys of 32 and values of 64; the queries' factor steps at every position;
     seventy experts (more than a wave's lanes) of which one is chosen, a wide shared expert; a recurrent layer of four
     heads of 64 x 64, run twice.
-X4: recurrent layers only (no pages at all), dense and routed.
+X4: recurrent layers only (no pages at all), dense and then routed (a router in the last layer moves its own place only).
 X5: attention layers only (no state slot at all), keys wider than values, one layer without a feed-forward.
 """
 import json
@@ -67,7 +67,7 @@ X3 = {"architecture": "Malinex", "vocab": 256, "width": 128, "max_positions": 51
                  _layer("gla", _x3_gla, _dense(72)), _layer("gla", _x3_gla, _dense(72), weights_of=1)]}
 X4 = {"architecture": "Malinex", "vocab": 150, "width": 80, "max_positions": 400, "norm": {"eps": 1e-6},
       "logit_scale": 0.125,
-      "layers": [_layer("gla", _gla(2, 32, 48, 16.0, 4), _moe(4, 3, 24, 24)), _layer("gla", _gla(5, 16, 16, 2.0, 7), _dense(64))]}
+      "layers": [_layer("gla", _gla(5, 16, 16, 2.0, 7), _dense(64)), _layer("gla", _gla(2, 32, 48, 16.0, 4), _moe(4, 3, 24, 24))]}
 X5 = {"architecture": "Malinex", "vocab": 1100, "width": 48, "max_positions": 320, "norm": {"eps": 1e-5},
       "logit_scale": 1.5,
       "layers": [_layer("attention", _attn(3, 3, 48, 16, 0.15, (1.0, 100)), _dense(64)),

@@ -134,17 +134,22 @@ def small_ff(f: torch.Tensor, up: torch.Tensor, down: torch.Tensor, act: Callabl
     return _r(act(_r(f @ up.T, round_to)), round_to) @ down.T
 
 
-def router(f: torch.Tensor, wr: torch.Tensor, correction: torch.Tensor, top: int, margins: Optional[List] = None):
+def router(f: torch.Tensor, wr: torch.Tensor, correction: torch.Tensor, top: int, margins: Optional[List] = None,
+           at_stake: float = 0.01):
     """-> (chosen [T, top], weights [T, top]): softmax over all experts; the choice goes by score + correction, the
     weights are the chosen scores themselves over their sum.  ``margins`` collects, per token, by how much the last
-    chosen expert beats the first that is not, as a fraction of the largest choice score."""
+    chosen expert beats the first that is not, as a fraction of its own choice score; a token whose last chosen
+    expert weighs less than ``at_stake`` counts as sure (margin 1): the other choice would change next to nothing."""
     s = torch.softmax(f @ wr.T, dim=-1)
-    c = torch.sort(s + correction, dim=-1, descending=True).values
-    if margins is not None and top < c.shape[1]:
-        margins.append((c[:, top - 1] - c[:, top]) / c[:, 0].abs().clamp_min(1e-30))
     chosen = torch.topk(s + correction, top, dim=-1).indices
     picked = torch.gather(s, 1, chosen)
-    return chosen, picked / (picked.sum(dim=-1, keepdim=True) + 1e-20)
+    weights = picked / (picked.sum(dim=-1, keepdim=True) + 1e-20)
+    if margins is not None and top < s.shape[1]:
+        c = torch.sort(s + correction, dim=-1, descending=True).values
+        gap = (c[:, top - 1] - c[:, top]) / c[:, top - 1].abs().clamp_min(1e-30)
+        last = torch.gather(weights, 1, torch.argmin(torch.gather(s + correction, 1, chosen), dim=-1, keepdim=True))[:, 0]
+        margins.append(torch.where(last < at_stake, torch.ones_like(gap), gap))
+    return chosen, weights
 
 
 def routed_ff(f: torch.Tensor, w: Mapping[str, torch.Tensor], p: str, mlp: Mapping, round_to=None,
@@ -270,7 +275,7 @@ def random_weights(cfg: Mapping, seed: int = 0, store: torch.dtype = torch.bfloa
         elif name == "pos":
             t = 0.5 * rnd()
         elif last == "router":
-            t = 3.0 * rnd() / math.sqrt(shape[-1])
+            t = 6.0 * rnd() / math.sqrt(shape[-1])
         else:
             t = rnd() / math.sqrt(shape[-1])
         out[name] = t.to(store)
