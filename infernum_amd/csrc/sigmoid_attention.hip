@@ -8,9 +8,13 @@
 //                        1 + coef ln(floor((p + 1) / every) + 1), queries into their own rows, keys and values into
 //                        their pages;
 //   ia_sigattn_generic   one wave per (token, head), fp32 throughout, keys 64 at a time in the order of their
-//                        positions: the 32-bit path and the plain twin of the matrix-core kernels.
+//                        positions: the 32-bit path and the plain twin of the matrix-core kernels;
+//   ia_sigattn_mfma      bf16 on the matrix cores: single tokens (the query heads of a key/value head side by side,
+//                        the keys in parts over workgroups and waves, joined in a fixed order) and portions of
+//                        prompts (a wave per 16 rows of a head).
 //
-// Pages: keys [num_pages, nkv, page_size, dim], values [num_pages, nkv, page_size, vdim]; block_tables[s, j / page_size]
+// Pages: keys [num_pages, nkv, page_size, dim], values transposed [num_pages, nkv, vdim, page_size] (four keys of
+// one value channel are 8 contiguous bytes, the operand of the second product); block_tables[s, j / page_size]
 // is the page of key j of request s.  A sum of weights has no reference point to move, so parts of the keys add up.
 #include "common.h"
 
@@ -57,7 +61,7 @@ __global__ __launch_bounds__(256) void sigattn_prepare_kernel(
   for (int i = tid; i < nv; i += 256) {
     const int g = i / vdim, c = i - g * vdim;
     const float x = to_float(row[nq + nk + i]) + (bv ? bv[i] : 0.f);
-    v_pages[(((size_t)page * nkv + g) * page_size + off) * vdim + c] = from_float<T>(x);
+    v_pages[(((size_t)page * nkv + g) * vdim + c) * page_size + off] = from_float<T>(x);
   }
 }
 
@@ -100,6 +104,7 @@ __global__ __launch_bounds__(64) void sigattn_generic_kernel(
   __shared__ float qs[SA_MAX_D];
   __shared__ float ps[64];
   __shared__ int rs[64];
+  __shared__ size_t vs[64];
   const int n = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
   const int s = token_seq[n];
   const int pos = positions[n];
@@ -116,10 +121,12 @@ __global__ __launch_bounds__(64) void sigattn_generic_kernel(
     const int j = j0 + lane;
     float p = 0.f;
     int row = 0;
+    size_t vat = 0;
     if (j <= pos) {
       const int page = bt[j / page_size];
       if ((unsigned)page < (unsigned)num_pages) {
         row = (page * nkv + g) * page_size + (j % page_size);
+        vat = ((size_t)page * nkv + g) * vdim * page_size + (j % page_size);
         const T* kr = k_pages + (size_t)row * dim;
         float dot = 0.f;
         for (int i = 0; i < dim; ++i) dot = fmaf(qs[i], to_float(kr[i]), dot);
@@ -131,15 +138,16 @@ __global__ __launch_bounds__(64) void sigattn_generic_kernel(
     }
     ps[lane] = p;
     rs[lane] = row;
+    vs[lane] = vat;
     __syncthreads();
     const int cnt = (pos - j0 + 1) < 64 ? (pos - j0 + 1) : 64;
     for (int jj = 0; jj < cnt; ++jj) {
-      const T* vr = v_pages + (size_t)rs[jj] * vdim;
+      const T* vr = v_pages + vs[jj];
       const float pj = ps[jj];
 #pragma unroll
       for (int c = 0; c < SA_MAX_D / 64; ++c) {
         const int i = lane + 64 * c;
-        if (i < vdim) acc[c] = fmaf(pj, to_float(vr[i]), acc[c]);
+        if (i < vdim) acc[c] = fmaf(pj, to_float(vr[(size_t)i * page_size]), acc[c]);
       }
     }
     __syncthreads();

@@ -1334,9 +1334,9 @@ def sigattn_prepare(proj: torch.Tensor, bq, bk, bv, wq: torch.Tensor, wk: Option
         _i32(slots, N, "sigattn_prepare slots")
         _dev(k_pages, v_pages)
         num_pages, ps = k_pages.shape[0], k_pages.shape[2]
-        _need(tuple(k_pages.shape) == (num_pages, nkv, ps, dim) and tuple(v_pages.shape) == (num_pages, nkv, ps, vdim)
+        _need(tuple(k_pages.shape) == (num_pages, nkv, ps, dim) and tuple(v_pages.shape) == (num_pages, nkv, vdim, ps)
               and k_pages.dtype == proj.dtype and v_pages.dtype == proj.dtype,
-              "sigattn_prepare: pages [P, nkv, page, dim] and [P, nkv, page, vdim] of the rows' dtype")
+              "sigattn_prepare: pages [P, nkv, page, dim] and [P, nkv, vdim, page] of the rows' dtype")
     _ok(_core().ia_sigattn_prepare(_p(proj), DTYPE_CODE[proj.dtype], int(proj.stride(0)), _p(bq), _p(bk), _p(bv), _p(wq),
                                    _p(wk), ctypes.c_float(eps), ctypes.c_float(temp_coef), int(temp_every),
                                    _p(positions), _p(slots), _p(q_out), _p(k_pages), _p(v_pages), N, nh, nkv, dim, vdim,
@@ -1349,7 +1349,7 @@ def _check_sigattn(q, k_pages, v_pages, gate, out, nh, nkv, dim, vdim, what):
     _rows(q, nh * dim, what + " queries")
     _dev(k_pages, v_pages, out)
     num_pages, ps = k_pages.shape[0], k_pages.shape[2]
-    _need(tuple(k_pages.shape) == (num_pages, nkv, ps, dim) and tuple(v_pages.shape) == (num_pages, nkv, ps, vdim)
+    _need(tuple(k_pages.shape) == (num_pages, nkv, ps, dim) and tuple(v_pages.shape) == (num_pages, nkv, vdim, ps)
           and k_pages.dtype == q.dtype and v_pages.dtype == q.dtype, what + ": pages of the queries' dtype and sizes")
     _need(tuple(out.shape) == (N, nh * vdim) and out.dtype == q.dtype, what + ": out [N, nh vdim]")
     if gate is not None:
@@ -1373,6 +1373,68 @@ def sigattn_generic(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tenso
                                    _p(token_seq), _p(positions), _p(block_tables), block_tables.shape[1], _p(r1), _p(r2),
                                    _p(pb), N, nh, nkv, dim, vdim, ps, num_pages, ctypes.c_float(scale), _stream()),
         "sigattn_generic")
+    return out
+
+
+def sigattn_mfma_available(dim: int, vdim: int) -> bool:
+    """Whether the matrix-core kernels of the sigmoid attention take these key and value sizes (their library is
+    built at its first use)."""
+    return dim in _build.SUPPORTED_HEAD_DIMS and vdim in _build.SUPPORTED_HEAD_DIMS
+
+
+def _sigattn(dim: int, vdim: int) -> ctypes.CDLL:
+    return load_library(f"sigattn_d{dim}_v{vdim}")
+
+
+def sigattn_decode_parts(batch: int, nh: int, nkv: int, max_len: int, device: Optional[torch.device] = None) -> int:
+    """Parts the keys of a single token are cut into by :func:`sigattn_decode`: enough workgroups (one per token,
+    group of up to 16 heads of a key/value head, and part) for about two a compute unit, no part shorter than the 64
+    keys that a workgroup's four waves take at a time, at most 64 parts."""
+    groups = batch * nkv * (-(-(nh // nkv) // 16))
+    wanted = -(-2 * compute_units(device) // max(groups, 1))
+    return max(1, min(wanted, -(-max_len // 64), 64))
+
+
+def sigattn_decode(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, gate: Optional[torch.Tensor],
+                   out: torch.Tensor, positions: torch.Tensor, block_tables: torch.Tensor, r1, r2, pb, nh: int, nkv: int,
+                   dim: int, vdim: int, scale: float, max_len: int, parts: Optional[int] = None) -> torch.Tensor:
+    """:func:`sigattn_generic` for B single tokens (row b: token b at positions[b], row b of the block tables) in bf16
+    on the matrix cores.  ``max_len`` bounds the positions (host side) and sets into how many parts the keys are cut."""
+    B, num_pages, ps = _check_sigattn(q, k_pages, v_pages, gate, out, nh, nkv, dim, vdim, "sigattn_decode")
+    _need(q.dtype == torch.bfloat16 and ps % 4 == 0, "sigattn_decode: bf16, and a page size that is a multiple of 4")
+    for t in (r1, r2, pb):
+        _f32(t, nh, "sigattn_decode per-head numbers")
+    _i32(positions, B, "sigattn_decode positions")
+    _need(block_tables.dtype == torch.int32 and block_tables.dim() == 2 and block_tables.is_contiguous()
+          and block_tables.shape[0] >= B and block_tables.shape[1] * ps >= max_len, "sigattn_decode: block tables")
+    parts = parts or sigattn_decode_parts(B, nh, nkv, max_len, out.device)
+    part = torch.empty(B * parts * nh * vdim, dtype=torch.float32, device=out.device) if parts > 1 else None
+    _ok(_sigattn(dim, vdim).ia_sigattn_decode(
+        _p(q), int(q.stride(0)), _p(k_pages), _p(v_pages), _p(gate), int(gate.stride(0)) if gate is not None else 0,
+        _p(out), _p(part), _p(positions), _p(block_tables), block_tables.shape[1], _p(r1), _p(r2), _p(pb), B, nh, nkv, ps,
+        num_pages, ctypes.c_float(scale), int(parts), _stream()), "sigattn_decode")
+    return out
+
+
+def sigattn_prefill(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, gate: Optional[torch.Tensor],
+                    out: torch.Tensor, seq_starts: torch.Tensor, seq_ctx: torch.Tensor, block_tables: torch.Tensor,
+                    tiles: torch.Tensor, num_tiles: int, r1, r2, pb, nh: int, nkv: int, dim: int, vdim: int,
+                    scale: float) -> torch.Tensor:
+    """:func:`sigattn_generic` for portions of prompts in bf16 on the matrix cores: request s has the rows
+    seq_starts[s] .. seq_starts[s + 1] - 1, seq_ctx[s] keys before them and row s of the block tables; tiles[i] =
+    (s, first row of a block of PREFILL_TILE_ROWS among the request's rows).  Rows of no tile are left alone."""
+    N, num_pages, ps = _check_sigattn(q, k_pages, v_pages, gate, out, nh, nkv, dim, vdim, "sigattn_prefill")
+    _need(q.dtype == torch.bfloat16 and ps % 4 == 0, "sigattn_prefill: bf16, and a page size that is a multiple of 4")
+    for t in (r1, r2, pb):
+        _f32(t, nh, "sigattn_prefill per-head numbers")
+    _dev(seq_starts, seq_ctx, tiles)
+    _need(seq_starts.dtype == torch.int32 and seq_ctx.dtype == torch.int32 and tiles.dtype == torch.int32
+          and tiles.is_contiguous() and tiles.numel() >= 2 * num_tiles, "sigattn_prefill: int32 starts, contexts and tiles")
+    _need(block_tables.dtype == torch.int32 and block_tables.dim() == 2 and block_tables.is_contiguous(), "sigattn_prefill: block tables")
+    _ok(_sigattn(dim, vdim).ia_sigattn_prefill(
+        _p(q), int(q.stride(0)), _p(k_pages), _p(v_pages), _p(gate), int(gate.stride(0)) if gate is not None else 0,
+        _p(out), _p(seq_starts), _p(seq_ctx), _p(block_tables), block_tables.shape[1], _p(tiles), int(num_tiles), _p(r1),
+        _p(r2), _p(pb), nh, nkv, ps, num_pages, ctypes.c_float(scale), _stream()), "sigattn_prefill")
     return out
 
 
@@ -1433,7 +1495,7 @@ def attention_mfma_available(d: int) -> bool:
 # standard error when the process ends (``profile_report`` gives it at any time).  The reference's switch of the
 # same name prints the time per operation of its graph executor (infernum-cpu/src/executor.rs:24-71).  Steps
 # are not recorded into HIP graphs meanwhile (a replayed launch has no call to bracket).
-_PROFILED = ("gemm_mfma_grouped", "norm_add", "activation", "latent_prepare", "gemm_heads", "router_topk", "moe_experts", "cast", "copy_pages", "gather_tokens", "words_from_host", "words_to_host", "embed", "add_rmsnorm", "residual_add", "rope_kv_append", "swiglu", "gemm_generic", "gemm_mfma",
+_PROFILED = ("sigattn_decode", "sigattn_prefill", "gemm_mfma_grouped", "norm_add", "activation", "latent_prepare", "gemm_heads", "router_topk", "moe_experts", "cast", "copy_pages", "gather_tokens", "words_from_host", "words_to_host", "embed", "add_rmsnorm", "residual_add", "rope_kv_append", "swiglu", "gemm_generic", "gemm_mfma",
              "gemm_library", "gemm_skinny", "gemm_skinny_rows", "attention_generic", "attention_decode", "attention_decode_rotating",
              "attention_prefill", "argmax", "repetition_penalty", "sample")
 _profile_on = False

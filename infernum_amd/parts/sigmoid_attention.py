@@ -9,7 +9,11 @@ factor.  There is no rotation.  Query head h reads key/value head h // (nh / nkv
 
 with nothing normalised over the keys, r1, r2, b numbers per head and gate = x Wg^T one number per token and head.
 Then the output projection.  One product makes q, k, v and the gates' logits; keys are kept [nkv, page, head_dim]
-and values [nkv, page, value_dim] per page.  Scores, the distance term, sigmoids and the sums over the keys are fp32.
+and values transposed, [nkv, value_dim, page], per page.  Scores, the distance term, sigmoids and the sums over the keys are fp32.
+
+In bf16, with head sizes that are multiples of 16 up to 256 and a page size that is a multiple of 4, the two products
+run on the matrix cores: one kernel for the step's single tokens (its first rows), one for its portions of prompts;
+every other case takes the plain kernel, one wave per token and head.
 """
 from __future__ import annotations
 
@@ -27,7 +31,7 @@ class SigmoidAttention(Mixer):
 
     def __init__(self, rt: Runtime, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int, value_dim: int,
                  scale: float, norm_eps: float, q_temp: Optional[Mapping[str, Any]] = None, biases: bool = True,
-                 gate: bool = True, distance_bias: bool = True, init_std: float = 0.02):
+                 gate: bool = True, distance_bias: bool = True, kernels: str = "auto", init_std: float = 0.02):
         """``q_temp`` {coef, every} or None; ``biases``: q, k and v have them; ``gate``: a sigmoid gate per token and
         head on the output; ``distance_bias``: the heads have r1, r2 (the term r1 ln(1 + r2 distance) taken off the
         score) and the number b added to it."""
@@ -45,11 +49,20 @@ class SigmoidAttention(Mixer):
         self.nq, self.nk, self.nv = self.nh * self.dim, self.nkv * self.dim, self.nkv * self.vdim
         self.row = self.nq + self.nk + self.nv + (self.nh if self.gate else 0)
         self.bq = self.bk = self.bv = self.r1 = self.r2 = self.pb = None
+        if kernels not in ("auto", "generic"):
+            raise ValueError("kernels must be 'auto' or 'generic'")
+        self.use_mfma = (kernels == "auto" and rt.kernels == "auto" and rt.dtype == torch.bfloat16
+                         and rt.device.type == "cuda" and K.sigattn_mfma_available(self.dim, self.vdim)
+                         and self.nq % 8 == 0 and self.row % 8 == 0)
 
     # ---- what it needs ---------------------------------------------------
     def cache_spec(self) -> CacheSpec:
         return CacheSpec("full", payload=(PageTensor("k", (self.nkv, self.dim), token_axis=1),
-                                          PageTensor("v", (self.nkv, self.vdim), token_axis=1)))
+                                          PageTensor("v", (self.nkv, self.vdim), token_axis=2)))
+
+    def step_needs(self) -> Dict[str, Any]:
+        # the matrix-core kernel for portions of prompts works on tiles of 64 query rows
+        return {"row_tiles": K.PREFILL_TILE_ROWS} if self.use_mfma else {}
 
     def weights(self) -> Dict[str, WeightSpec]:
         H, init, small = self.hidden_size, ("normal", self.init_std), dict(follows_compute_dtype=False)
@@ -120,19 +133,56 @@ class SigmoidAttention(Mixer):
         program.pending = emit_linear(program, out, N, self.w_o, rt.dtype, None, True, "sigattn.o", "sigattn.o_proj")
 
     def emit_attend(self, program, view: CacheView, q, gate, out) -> None:
-        from ..engine.program import STREAM
+        from ..engine.program import STREAM, Guard
         k, v, g = view.k_pages, view.v_pages, view.group
-        program.op("core", "ia_sigattn_generic", [q, self.nq, k, v, gate, self.row if gate is not None else 0, out,
-                                                  program.act_code, program.token_seq, program.positions,
-                                                  program.block_table(g), program.bt_cols(g), self.r1, self.r2, self.pb,
-                                                  program.N, self.nh, self.nkv, self.dim, self.vdim, int(k.shape[2]),
-                                                  int(k.shape[0]), float(self.scale), STREAM])
+        ps, num_pages = int(k.shape[2]), int(k.shape[0])
+        gate_stride = self.row if gate is not None else 0
+        bt, bt_cols = program.block_table(g), program.bt_cols(g)
+        if not (self.use_mfma and ps % 4 == 0):
+            program.op("core", "ia_sigattn_generic", [q, self.nq, k, v, gate, gate_stride, out, program.act_code,
+                                                      program.token_seq, program.positions, bt, bt_cols, self.r1, self.r2,
+                                                      self.pb, program.N, self.nh, self.nkv, self.dim, self.vdim, ps,
+                                                      num_pages, float(self.scale), STREAM])
+            return
+        lib = K._sigattn(self.dim, self.vdim)
+        records = program.T + 1024          # tokens x parts of their keys: what fills the GPU, or the tokens themselves
+        part = program.buffer("sigattn.part", records * self.nh * self.vdim * 4)
+        nh, nkv, dev = self.nh, self.nkv, self.rt.device
+
+        def parts_of_the_keys(ctx: StepContext) -> int:
+            nd = ctx.num_decode
+            if nd == 0:
+                return 1
+            if ctx.block_tables[g].shape[1] * ps < ctx.max_total_len:
+                raise K.KernelError("sigmoid_attention: the block tables are narrower than the longest request")
+            n = K.sigattn_decode_parts(nd, nh, nkv, ctx.max_total_len, dev)
+            return max(1, min(n, records // nd))
+        parts = program.scalar(("sigmoid_attention: parts of the keys", nh, nkv, g, ps), parts_of_the_keys)
+        tiles, num_tiles = program.row_tiles(K.PREFILL_TILE_ROWS)
+        program.op(lib, "ia_sigattn_decode", [q, self.nq, k, v, gate, gate_stride, out, part, program.positions, bt,
+                                              bt_cols, self.r1, self.r2, self.pb, program.ND, nh, nkv, ps, num_pages,
+                                              float(self.scale), parts, STREAM], Guard.between(program.ND, 1))
+        program.op(lib, "ia_sigattn_prefill", [q, self.nq, k, v, gate, gate_stride, out, program.seq_starts,
+                                               program.seq_ctx, bt, bt_cols, tiles, num_tiles, self.r1, self.r2, self.pb,
+                                               nh, nkv, ps, num_pages, float(self.scale), STREAM],
+                   Guard.between(program.NP, 1))
 
     def attend(self, q: torch.Tensor, gate: Optional[torch.Tensor], out: torch.Tensor, ctx: StepContext,
                cache: CacheView) -> None:
-        K.sigattn_generic(q, cache.k_pages, cache.v_pages, gate, out, ctx.token_seq, ctx.positions,
-                          ctx.block_tables[cache.group], self.r1, self.r2, self.pb, self.nh, self.nkv, self.dim, self.vdim,
-                          self.scale)
+        bt = ctx.block_tables[cache.group]
+        if not (self.use_mfma and cache.k_pages.shape[2] % 4 == 0):
+            K.sigattn_generic(q, cache.k_pages, cache.v_pages, gate, out, ctx.token_seq, ctx.positions, bt, self.r1,
+                              self.r2, self.pb, self.nh, self.nkv, self.dim, self.vdim, self.scale)
+            return
+        nd = ctx.num_decode
+        if nd > 0:
+            K.sigattn_decode(q[:nd], cache.k_pages, cache.v_pages, gate[:nd] if gate is not None else None, out[:nd],
+                             ctx.positions[:nd], bt, self.r1, self.r2, self.pb, self.nh, self.nkv, self.dim, self.vdim,
+                             self.scale, ctx.max_total_len)
+        if ctx.num_seqs > nd:
+            tiles, num_tiles = ctx.row_tiles(K.PREFILL_TILE_ROWS)
+            K.sigattn_prefill(q, cache.k_pages, cache.v_pages, gate, out, ctx.seq_starts, ctx.seq_ctx, bt, tiles,
+                              num_tiles, self.r1, self.r2, self.pb, self.nh, self.nkv, self.dim, self.vdim, self.scale)
 
 
 register_part("mixer", "sigmoid_attention", SigmoidAttention)

@@ -258,7 +258,7 @@ def test_a_state_that_reaches_hundreds_of_tokens_back(dtype):
     x0[3] = 0.0
     tol = _tol(dtype, want, lambda: PM.gla_mixer(x.double(), w, "", m, EPS, round_to=torch.bfloat16))
     shows = (want[-8:] - PM.gla_mixer(x0.double(), w, "", m, EPS)[-8:]).abs().max() / want.pow(2).mean().sqrt()
-    assert shows > 10 * tol, (shows, tol)
+    assert shows > 5 * tol, (shows, tol)
     for cuts in ([T], [300, T - 305] + [1] * 5, [3, 1, 200, T - 204]):
         steps = Steps([(None, mixer.state_spec())], rt, slots=2)
         got = _run_mixer(mixer, steps, x, cuts, rt)
@@ -287,26 +287,91 @@ def test_sigmoid_attention_alone(dtype, m, W, T, ps):
         assert rel_err(got.to(rt.dtype), want) <= tol, cuts[:3]
 
 
+@pytest.mark.parametrize("nh,nkv,dim,vdim,ps", [(4, 2, 16, 32, 4), (20, 1, 32, 64, 12), (3, 3, 48, 16, 16), (8, 2, 128, 64, 8),
+                                                (2, 1, 128, 128, 20)])
+def test_sigmoid_attention_on_the_matrix_cores_against_the_plain_kernel(nh, nkv, dim, vdim, ps):
+    """The kernels for single tokens (whole, and with the keys cut into 2, 5 and 64 parts) and for portions of
+    prompts (rows of 1 to 150 behind 0 to 130 keys) give what the plain kernel gives on the same pages, of sizes that
+    are and are not powers of two; places of the pages that no request holds are NaN."""
+    from infernum_amd.kernels import api as K
+    g = torch.Generator().manual_seed(nh * dim + ps)
+    lens = [1, 2, 17, 64, 65, 200, 333]
+    per = max(-(-n // ps) for n in lens)
+    P = len(lens) * per + 3
+    perm = torch.randperm(P, generator=g).tolist()
+    bt = torch.full((len(lens), per), -1, dtype=torch.int32)
+    k = torch.full((P, nkv, ps, dim), float("nan"))
+    v = torch.full((P, nkv, vdim, ps), float("nan"))
+    for b, n in enumerate(lens):
+        for i in range(-(-n // ps)):
+            page = perm.pop()
+            bt[b, i] = page
+            m = min(ps, n - i * ps)
+            k[page, :, :m] = torch.randn(nkv, m, dim, generator=g)
+            v[page, :, :, :m] = torch.randn(nkv, vdim, m, generator=g)
+    k, v, bt = k.to(DEV).to(torch.bfloat16), v.to(DEV).to(torch.bfloat16), bt.to(DEV)
+    r1, r2, pb = (torch.rand(nh, generator=g) * 0.8 + 0.2).to(DEV), (torch.rand(nh, generator=g) * 0.45 + 0.05).to(DEV), \
+        (-1 - 2 * torch.rand(nh, generator=g)).to(DEV)
+    scale = 0.5 / math.sqrt(dim)
+
+    def rows(N):
+        q = torch.randn(N, nh * dim + 8, generator=g).to(DEV).to(torch.bfloat16)[:, :nh * dim]
+        gate = torch.randn(N, nh + 3, generator=g).to(DEV).to(torch.bfloat16)[:, 3:]
+        return q, gate, torch.empty((N, nh * vdim), dtype=torch.bfloat16, device=DEV), \
+            torch.full((N, nh * vdim), 7.0, dtype=torch.bfloat16, device=DEV)
+    # single tokens: the last place of every request
+    B = len(lens)
+    q, gate, want, got = rows(B)
+    pos, seq = torch.tensor([n - 1 for n in lens], dtype=torch.int32, device=DEV), torch.arange(B, dtype=torch.int32, device=DEV)
+    K.sigattn_generic(q, k, v, gate, want, seq, pos, bt, r1, r2, pb, nh, nkv, dim, vdim, scale)
+    assert torch.isfinite(want).all()
+    for parts in (1, 2, 5, 64, None):
+        got.fill_(7.0)
+        K.sigattn_decode(q, k, v, gate, got, pos, bt, r1, r2, pb, nh, nkv, dim, vdim, scale, max(lens), parts)
+        assert rel_err(got, want.float().cpu()) <= PART_TOL["bfloat16"], parts
+    # portions: the last rows of every request, of many lengths
+    qlens = [1, 2, 16, 64, 65, 70, 150]
+    ctx = [n - m for n, m in zip(lens, qlens)]
+    starts = [0]
+    for m in qlens:
+        starts.append(starts[-1] + m)
+    q, gate, want, got = rows(starts[-1])
+    seq = torch.cat([torch.full((m,), b, dtype=torch.int32) for b, m in enumerate(qlens)]).to(DEV)
+    pos = torch.cat([torch.arange(c, c + m, dtype=torch.int32) for c, m in zip(ctx, qlens)]).to(DEV)
+    tiles = torch.tensor([(b, f) for b, m in enumerate(qlens) for f in range(0, m, K.PREFILL_TILE_ROWS)], dtype=torch.int32).to(DEV)
+    K.sigattn_generic(q, k, v, gate, want, seq, pos, bt, r1, r2, pb, nh, nkv, dim, vdim, scale)
+    K.sigattn_prefill(q, k, v, gate, got, torch.tensor(starts, dtype=torch.int32, device=DEV),
+                      torch.tensor(ctx, dtype=torch.int32, device=DEV), bt, tiles, tiles.shape[0], r1, r2, pb, nh, nkv, dim,
+                      vdim, scale)
+    assert torch.isfinite(want).all() and rel_err(got, want.float().cpu()) <= PART_TOL["bfloat16"]
+    # a key that is needed and has no page: NaN in its request's rows, never a stray read
+    bt[5, 1] = -1
+    K.sigattn_decode(q[:B], k, v, gate[:B], got[:B], torch.tensor([n - 1 for n in lens], dtype=torch.int32, device=DEV), bt, r1,
+                     r2, pb, nh, nkv, dim, vdim, scale, max(lens), 1)
+    assert torch.isnan(got[5]).all() and torch.isfinite(got[:5]).all() and torch.isfinite(got[6]).all()
+
+
 def _standing_out(dtype, T, star, first):
-    """A mixer (two heads over one key head of 64, values of 32) and inputs in which every query from row ``first`` on
+    """A mixer (two heads over one key head of 128, values of 32) and inputs in which every query from row ``first`` on
     points at token ``star``'s key: wherever that key is visible its weight is near one, and every other key's is
     near zero (a low number b on every score), so the output is the star's value or nothing.  The keys come from a
     projection that does not see the direction u; the queries see u alone and answer it with the star's key."""
     rt = runtime(dtype)
-    W, d = 48, 64
-    m = MM._attn(2, 1, d, 32, 0.5, (0.25, 7))
+    W, d = 48, 128
+    m = MM._attn(2, 1, d, 32, 0.3)
     w = _mixer_weights("attention", m, W, 1)
     g = torch.Generator().manual_seed(4)
     u = torch.randn(W, generator=g).double()
     u /= u.norm()
     w["k"] = (w["k"] - (w["k"] @ u)[:, None] * u[None, :]).to(torch.bfloat16).double()
+    w["k.b"] = torch.zeros(d, dtype=torch.float64)        # a bias would be a part that all keys share with the star's
     x = _x(T, W, dtype, 3, 1.0).double()
     x = x - (x @ u)[:, None] * u[None, :]
     k = PM.rms_norm(x @ w["k"].t() + w["k.b"], w["k.norm"], EPS)
     w["q"] = torch.cat([torch.outer(k[star], u)] * 2).to(torch.bfloat16).double()
     w["q.b"] = (0.3 * torch.randn(2 * d, generator=g)).to(torch.bfloat16).double()
     w["q.norm"] = torch.ones(2 * d, dtype=torch.float64)
-    w["pb"] = torch.full((2,), -22.0, dtype=torch.float64)
+    w["pb"] = torch.full((2,), -26.0, dtype=torch.float64)
     x[first:] += 4.0 * u
     x = x.float()
     if dtype == "bfloat16":
@@ -326,7 +391,7 @@ def test_a_key_that_stands_out_at_the_causal_edge_and_at_page_borders(dtype, sta
     want = PM.attention_mixer(x.double(), w, "", m, EPS)
     rms = want.pow(2).mean().sqrt()
     tol = _tol(dtype, want, lambda: PM.attention_mixer(x.double(), w, "", m, EPS, round_to=torch.bfloat16))
-    assert want[:star].abs().max() < 1e-3 * rms and want[star].abs().max() > 0.3 * rms     # nothing, then the value
+    assert want[:star].abs().max() < 1e-2 * rms and want[star].abs().max() > 0.3 * rms     # nothing, then the value
     for cuts in ([T], [star - 1] + [1] * 4 + [T - star - 3], [star, T - star], [star + 1, T - star - 1], [2] * (T // 2)):
         steps = Steps([(mixer.cache_spec(), None)], rt, page_size=4, num_pages=16, poison=True)
         got = _run_mixer(mixer, steps, x, [c for c in cuts if c], rt)
