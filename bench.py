@@ -525,6 +525,61 @@ def rogizen_active_params(size: dict) -> int:
     return (n // 4) * attention + (n - n // 4) * ssm + n * 3 * W * size["ff"] + 2 * W * W + size["vocab"] * W
 
 
+# ---- the Malinex design beside the Llama decoder at equal sizes -------------------------------------------------
+# Eight layers of one width: three layers of gated linear attention (heads of 128 keys x 128 values, a decay per key
+# channel through a matrix pair of rank 64), then a layer of attention with sigmoid weights and a distance term (heads
+# of 128 over 4 key/value heads, the queries' factor stepping every 512 positions), twice.  Odd layers have a dense
+# feed-forward of one and a half times the twin's inner size (two matrices against the twin's three), even layers eight
+# experts of a third of that, two chosen, and a shared expert of the same size: the same weights a token.  The Llama
+# twin has the same width, layers, vocabulary, heads and feed-forward weights a token.
+MALINEX_SIZES = {
+    "2k": dict(width=2048, layers=8, vocab=32000, ff=5504, heads=16, kv_heads=4, dim=128, experts=8, top=2, rank=64),
+    "4k": dict(width=4096, layers=8, vocab=32000, ff=9600, heads=32, kv_heads=8, dim=128, experts=8, top=2, rank=64),
+}
+
+
+def malinex_configs(size: dict):
+    from infernum_amd.config import LlamaConfig
+    from infernum_amd.config.malinex import MalinexConfig
+    d, ff2 = size["dim"], size["ff"] * 3 // 2
+    attention = {"heads": size["heads"], "kv_heads": size["kv_heads"], "dim": d, "vdim": d, "scale": d ** -0.5,
+                 "q_temp": {"coef": 0.1, "every": 512}}
+    gla = {"heads": size["heads"], "dim": d, "vdim": d, "tau": 16.0, "rank": size["rank"]}
+    dense = {"kind": "dense", "ff": ff2}
+    moe = {"kind": "moe", "router": {"experts": size["experts"], "top": size["top"]}, "expert": {"ff": ff2 // 3},
+           "shared": {"ff": ff2 // 3}}
+    mal = MalinexConfig.from_dict({
+        "architecture": "Malinex", "vocab": size["vocab"], "width": size["width"], "max_positions": 8192,
+        "norm": {"eps": 1e-6}, "logit_scale": 0.25,
+        "layers": [{"type": "attention" if i % 4 == 3 else "gla", "mixer": attention if i % 4 == 3 else gla,
+                    "mlp": dense if i % 2 else moe} for i in range(size["layers"])]})
+    llama = LlamaConfig.from_dict(dict(
+        model_type="llama", num_hidden_layers=size["layers"], hidden_size=size["width"],
+        num_attention_heads=size["heads"], num_key_value_heads=size["kv_heads"], intermediate_size=size["ff"],
+        vocab_size=size["vocab"], rope_theta=10000.0, rms_norm_eps=1e-6, tie_word_embeddings=True,
+        max_position_embeddings=8192))
+    return mal, llama
+
+
+def malinex_active_params(size: dict) -> int:
+    """Weights that a token multiplies with in the Malinex model of these sizes (the head and the branches' gates
+    included)."""
+    W, n, d, ff2 = size["width"], size["layers"], size["dim"], size["ff"] * 3 // 2
+    hd = size["heads"] * d
+    gla = W * 4 * hd + size["rank"] * (W + hd) + hd * W
+    attention = W * (hd + 2 * size["kv_heads"] * d + size["heads"]) + hd * W
+    dense = 2 * W * ff2
+    moe = W * size["experts"] + (size["top"] + 1) * 2 * W * (ff2 // 3)
+    gates = 2 * W * W
+    return (n // 4) * attention + (n - n // 4) * gla + (n // 2) * dense + (n - n // 2) * moe + n * gates + size["vocab"] * W
+
+
+def malinex_bench(a) -> int:
+    batches = [int(b) for b in a.malinex_batches.split(",") if b]
+    return beside_llama_bench(a, "Malinex", [(n, MALINEX_SIZES[n]) for n in a.malinex.split(",")], malinex_configs,
+                              malinex_active_params, batches)
+
+
 def nesilorn_bench(a) -> int:
     batches = [int(b) for b in a.nesilorn_batches.split(",") if b]
     return beside_llama_bench(a, "Nesilorn", [(n, NESILORN_SIZES[n]) for n in a.nesilorn.split(",")], nesilorn_configs,
@@ -632,6 +687,10 @@ def main() -> int:
                          "Llama decoder at equal sizes instead: prefill and decode of each (a JSON line of its own); "
                          "sizes: 2k, 4k or both with a comma")
     ap.add_argument("--rogizen-batches", default="8,64", help="decode batches of --rogizen")
+    ap.add_argument("--malinex", default="", metavar="SIZES",
+                    help="the Malinex design (gated linear attention, attention with sigmoid weights, routed experts) beside "
+                         "the Llama decoder at equal sizes: names of " + ", ".join(MALINEX_SIZES) + " with commas")
+    ap.add_argument("--malinex-batches", default="8,64", help="decode batches of --malinex")
     a = ap.parse_args()
     if a.gpus != 1:
         print(f"bench.py measures one GPU: this engine has no multi-GPU path (asked for --gpus {a.gpus})")
@@ -639,6 +698,8 @@ def main() -> int:
 
     if a.nesilorn:
         return nesilorn_bench(a)
+    if a.malinex:
+        return malinex_bench(a)
     if a.rogizen:
         return rogizen_bench(a)
     if a.decode_kernels:

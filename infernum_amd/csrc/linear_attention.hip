@@ -6,6 +6,11 @@
 //
 //   ia_gla_scan         the recurrence token after token for the rows of every request of a step, from the request's
 //                       state slot, which it leaves moved on;
+//   ia_gla_chunked      the same for portions of prompts cut into tiles of GLA_TILE rows that run side by side: every
+//                       tile but a request's last first runs from a zero state and leaves what it adds, U, and the
+//                       product D of its decays; a second kernel walks a request's tiles, S <- diag(D) S + U, and
+//                       leaves every tile the state before it; then every tile runs from that state and writes its
+//                       rows, the last one the request's slot.  All of it fp32, as the recurrence itself;
 //   ia_head_norm_gate   norm per head, weight, silu(gate), rounded once into the activations' type.
 //
 // The state of a head is kept in slices of GLA_PW value columns: slot[head][slice][n][GLA_PW], so that the workgroup
@@ -16,6 +21,7 @@
 #define GLA_PW 16        // value columns of a workgroup's slice
 #define GLA_PARTS 16     // the key channels are dealt out over so many groups of threads
 #define GLA_TB 8         // tokens whose rows are staged together
+#define GLA_TILE 64      // rows of a tile of ia_gla_chunked
 
 __host__ __device__ inline int gla_slices(int vdim) { return (vdim + GLA_PW - 1) / GLA_PW; }
 
@@ -24,32 +30,59 @@ __device__ __forceinline__ float gla_log_sigmoid(float z) {
   return z >= 0.f ? -log1pf(expf(-z)) : z - log1pf(expf(z));
 }
 
-// grid (heads, requests, slices), 256 threads: thread (part, p) keeps S[n][p] for n = part, part + 16, ... in registers.
-template <typename T, int KMAX>
+// The record of the tile that begins at row r0 of request s: the tiles of the requests from ``first_request`` on,
+// counted in the order of the requests and their rows, whatever the order of the list of tiles.
+__device__ __forceinline__ int gla_record(const int* __restrict__ seq_starts, int first_request, int s, int r0) {
+  int before = 0;
+  for (int r = first_request; r < s; ++r) before += (seq_starts[r + 1] - seq_starts[r] + GLA_TILE - 1) / GLA_TILE;
+  return before + r0 / GLA_TILE;
+}
+
+// grid (heads, requests or tiles, slices), 256 threads: thread (part, p) keeps S[n][p] for n = part, part + 16, ...
+// in registers.  MODE 0: a request's rows from its slot, which is left moved on.  MODE 1: a tile (not a request's
+// last) from a zero state; no rows are written, the state goes to the tile's record and the product of the decays
+// to ``decay``.  MODE 2: a tile from its record; a request's last tile leaves the state in the slot.
+template <typename T, int KMAX, int MODE>
 __global__ __launch_bounds__(256) void gla_scan_kernel(
     const T* __restrict__ proj, int proj_stride, int q_col, int k_col, int v_col, const float* __restrict__ z,
     int z_stride, const float* __restrict__ z_bias, float inv_tau, float q_scale, float* __restrict__ state,
     long state_stride, float* __restrict__ out, const int* __restrict__ seq_starts, const int* __restrict__ state_slots,
-    int nh, int dim, int vdim) {
+    int nh, int dim, int vdim, const int* __restrict__ tiles, int first_request, float* __restrict__ records,
+    long record_stride, float* __restrict__ decay) {
   extern __shared__ float lds[];
   float* qs = lds;                                   // [TB][dim]
   float* ks = qs + GLA_TB * dim;                     // [TB][dim]
   float* as = ks + GLA_TB * dim;                     // [TB][dim]  alpha
   float* vs = as + GLA_TB * dim;                     // [TB][PW]
   float* ysum = vs + GLA_TB * GLA_PW;                // [TB][PARTS][PW]
-  const int hd = blockIdx.x, s = blockIdx.y, slice = blockIdx.z;
-  const int first = seq_starts[s], count = seq_starts[s + 1] - first;
+  const int hd = blockIdx.x, slice = blockIdx.z;
+  const int s = MODE == 0 ? blockIdx.y : tiles[2 * blockIdx.y];
+  int first = seq_starts[s], count = seq_starts[s + 1] - first;
+  bool last = true;
+  int record = 0;
+  if (MODE != 0) {
+    const int r0 = tiles[2 * blockIdx.y + 1];
+    last = r0 + GLA_TILE >= count;
+    if (MODE == 2 || !last) record = gla_record(seq_starts, first_request, s, r0);
+    first += r0;
+    count = last ? count - r0 : GLA_TILE;
+    if (MODE == 1 && last) return;
+  }
   if (count <= 0) return;
   const int tid = threadIdx.x;
   const int p = tid % GLA_PW, part = tid / GLA_PW;
   const int col = slice * GLA_PW + p;
   const int slices = gla_slices(vdim);
-  float* S = state + (size_t)state_slots[s] * state_stride + ((size_t)hd * slices + slice) * dim * GLA_PW;
+  const size_t within = ((size_t)hd * slices + slice) * dim * GLA_PW;
+  float* S = state + (size_t)state_slots[s] * state_stride + within;
+  float* R = MODE == 0 ? S : records + (size_t)record * record_stride + within;
+  float dprod[MODE == 1 ? KMAX : 1];
   float reg[KMAX];
 #pragma unroll
   for (int c = 0; c < KMAX; ++c) {
     const int n = part + c * GLA_PARTS;
-    reg[c] = n < dim ? S[(size_t)n * GLA_PW + p] : 0.f;
+    reg[c] = (MODE != 1 && n < dim) ? R[(size_t)n * GLA_PW + p] : 0.f;
+    if constexpr (MODE == 1) dprod[c] = 1.f;
   }
   for (int t0 = 0; t0 < count; t0 += GLA_TB) {
     const int nt = count - t0 < GLA_TB ? count - t0 : GLA_TB;
@@ -79,11 +112,13 @@ __global__ __launch_bounds__(256) void gla_scan_kernel(
         const int n = part + c * GLA_PARTS;
         if (n < dim) {
           reg[c] = __builtin_fmaf(at[n], reg[c], kt[n] * v);
-          acc = __builtin_fmaf(reg[c], qt[n], acc);
+          if constexpr (MODE == 1) dprod[c] *= at[n];
+          else acc = __builtin_fmaf(reg[c], qt[n], acc);
         }
       }
-      ysum[(t * GLA_PARTS + part) * GLA_PW + p] = acc;
+      if (MODE != 1) ysum[(t * GLA_PARTS + part) * GLA_PW + p] = acc;
     }
+    if (MODE == 1) continue;
     __syncthreads();
     for (int i = tid; i < nt * GLA_PW; i += 256) {
       const int t = i / GLA_PW, pp = i - t * GLA_PW;
@@ -94,10 +129,43 @@ __global__ __launch_bounds__(256) void gla_scan_kernel(
       if (c < vdim) out[(size_t)(first + t0 + t) * ((size_t)nh * vdim) + (size_t)hd * vdim + c] = y;
     }
   }
+  if (MODE == 2 && !last) return;
+  float* W = MODE == 1 ? R : S;
 #pragma unroll
   for (int c = 0; c < KMAX; ++c) {
     const int n = part + c * GLA_PARTS;
-    if (n < dim) S[(size_t)n * GLA_PW + p] = reg[c];
+    if (n < dim) {
+      W[(size_t)n * GLA_PW + p] = reg[c];
+      if constexpr (MODE == 1) if (p == 0 && slice == 0) decay[((size_t)record * nh + hd) * dim + n] = dprod[c];
+    }
+  }
+}
+
+// grid (heads x slices, tiles), 256 threads; the workgroup of a request's first tile walks the request's tiles: the
+// record of a tile holds what the tile adds when it comes and the state before the tile when it goes.
+__global__ __launch_bounds__(256) void gla_chain_kernel(const float* __restrict__ state, long state_stride,
+                                                        const int* __restrict__ seq_starts,
+                                                        const int* __restrict__ state_slots, const int* __restrict__ tiles,
+                                                        int first_request, float* __restrict__ records, long record_stride,
+                                                        const float* __restrict__ decay, int nh, int dim, int slices) {
+  const int i = blockIdx.y;
+  if (tiles[2 * i + 1] != 0) return;
+  const int s = tiles[2 * i], rows = seq_starts[s + 1] - seq_starts[s];
+  const int hs = blockIdx.x, hd = hs / slices;
+  const size_t within = (size_t)hs * dim * GLA_PW;
+  const float* S0 = state + (size_t)state_slots[s] * state_stride + within;
+  const int first = gla_record(seq_starts, first_request, s, 0);
+  for (int e = threadIdx.x; e < dim * GLA_PW; e += 256) {
+    const int n = e / GLA_PW;
+    float S = S0[e];
+    int j = first;
+    for (int r0 = 0; r0 < rows; r0 += GLA_TILE, ++j) {
+      float* at = records + (size_t)j * record_stride + within + e;
+      const bool last = r0 + GLA_TILE >= rows;
+      const float U = last ? 0.f : *at;
+      *at = S;
+      if (!last) S = __builtin_fmaf(decay[((size_t)j * nh + hd) * dim + n], S, U);
+    }
   }
 }
 
@@ -123,9 +191,10 @@ extern "C" int ia_gla_scan(const void* proj, int code, int proj_stride, int q_co
   const size_t lds = sizeof(float) * ((size_t)3 * GLA_TB * dim + GLA_TB * GLA_PW + (size_t)GLA_TB * GLA_PARTS * GLA_PW);
   if (lds > 64 * 1024) return IA_ERR_UNSUPPORTED;
 #define IA_GLA(T, KM)                                                                                                  \
-  gla_scan_kernel<T, KM><<<grid, 256, lds, stream>>>((const T*)proj, proj_stride, q_col, k_col, v_col, z, z_stride,    \
-                                                     z_bias, 1.0f / tau, q_scale, state, state_stride, out, seq_starts, \
-                                                     state_slots, nh, dim, vdim)
+  gla_scan_kernel<T, KM, 0><<<grid, 256, lds, stream>>>((const T*)proj, proj_stride, q_col, k_col, v_col, z, z_stride, \
+                                                        z_bias, 1.0f / tau, q_scale, state, state_stride, out,         \
+                                                        seq_starts, state_slots, nh, dim, vdim, nullptr, 0, nullptr,   \
+                                                        0, nullptr)
 #define IA_GLA_K(T)                       \
   do {                                    \
     if (per <= 4) IA_GLA(T, 4);           \
@@ -136,6 +205,57 @@ extern "C" int ia_gla_scan(const void* proj, int code, int proj_stride, int q_co
   if (code == IA_F32) IA_GLA_K(float);
   else if (code == IA_BF16) IA_GLA_K(bf16_t);
   else return IA_ERR_BAD_ARG;
+#undef IA_GLA_K
+#undef IA_GLA
+  IA_LAUNCH_CHECK();
+  return IA_OK;
+}
+
+// The recurrence of ia_gla_scan for the requests that the tiles name: tiles[i] = (request, first row of a tile of
+// GLA_TILE among the request's rows) in any order, every tile of the requests first_request .. (and of no other)
+// once.  records: fp32 [num_tiles, record_stride >= ia_gla_state_floats]; decay: fp32 [num_tiles, nh, dim].
+extern "C" int ia_gla_chunked(const void* proj, int code, int proj_stride, int q_col, int k_col, int v_col, const float* z,
+                              int z_stride, const float* z_bias, float tau, float q_scale, float* state,
+                              long state_stride, float* out, const int* seq_starts, const int* state_slots,
+                              const int* tiles, int num_tiles, int first_request, float* records, long record_stride, float* decay, int nh,
+                              int dim, int vdim, hipStream_t stream) {
+  if (num_tiles == 0) return IA_OK;
+  if (!proj || !z || !state || !out || !seq_starts || !state_slots || !tiles || !records || !decay || num_tiles < 0 || first_request < 0 ||
+      nh <= 0 || dim <= 0 || vdim <= 0 || !(tau > 0.f) || q_col < 0 || k_col < 0 || v_col < 0 ||
+      proj_stride < q_col + nh * dim || proj_stride < k_col + nh * dim || proj_stride < v_col + nh * vdim ||
+      z_stride < nh * dim || state_stride < ia_gla_state_floats(nh, dim, vdim) ||
+      record_stride < ia_gla_state_floats(nh, dim, vdim))
+    return IA_ERR_BAD_ARG;
+  const int per = (dim + GLA_PARTS - 1) / GLA_PARTS;
+  const int slices = gla_slices(vdim);
+  if (per > 32 || num_tiles > 65535 || slices > 65535) return IA_ERR_UNSUPPORTED;
+  const dim3 grid((unsigned)nh, (unsigned)num_tiles, (unsigned)slices);
+  const size_t lds = sizeof(float) * ((size_t)3 * GLA_TB * dim + GLA_TB * GLA_PW + (size_t)GLA_TB * GLA_PARTS * GLA_PW);
+  if (lds > 64 * 1024) return IA_ERR_UNSUPPORTED;
+#define IA_GLA(T, KM, MODE)                                                                                        \
+  gla_scan_kernel<T, KM, MODE><<<grid, 256, lds, stream>>>(                                                        \
+      (const T*)proj, proj_stride, q_col, k_col, v_col, z, z_stride, z_bias, 1.0f / tau, q_scale, state,           \
+      state_stride, out, seq_starts, state_slots, nh, dim, vdim, tiles, first_request, records, record_stride, decay)
+#define IA_GLA_K(T, MODE)                       \
+  do {                                          \
+    if (per <= 4) IA_GLA(T, 4, MODE);           \
+    else if (per <= 8) IA_GLA(T, 8, MODE);      \
+    else if (per <= 16) IA_GLA(T, 16, MODE);    \
+    else IA_GLA(T, 32, MODE);                   \
+  } while (0)
+#define IA_GLA_T(MODE)                             \
+  do {                                             \
+    if (code == IA_F32) IA_GLA_K(float, MODE);     \
+    else IA_GLA_K(bf16_t, MODE);                   \
+  } while (0)
+  if (code != IA_F32 && code != IA_BF16) return IA_ERR_BAD_ARG;
+  IA_GLA_T(1);
+  IA_LAUNCH_CHECK();
+  gla_chain_kernel<<<dim3((unsigned)(nh * slices), (unsigned)num_tiles), 256, 0, stream>>>(
+      state, state_stride, seq_starts, state_slots, tiles, first_request, records, record_stride, decay, nh, dim, slices);
+  IA_LAUNCH_CHECK();
+  IA_GLA_T(2);
+#undef IA_GLA_T
 #undef IA_GLA_K
 #undef IA_GLA
   IA_LAUNCH_CHECK();
@@ -188,4 +308,5 @@ extern "C" int ia_head_norm_gate(const float* o, const void* gate, int code, int
 
 #include "op_call.h"
 IA_OP(ia_gla_scan)
+IA_OP(ia_gla_chunked)
 IA_OP(ia_head_norm_gate)

@@ -221,7 +221,8 @@ __global__ __launch_bounds__(64) void sigattn_join_kernel(const float* __restric
 // ------------------------------------------------------------------------ portions of prompts
 // 256 threads; a workgroup is one tile (request, first row) of 64 rows and one query head; wave w takes the rows
 // first + 16 w .. + 15.  Workgroups are numbered so that the heads of one tile follow each other (they go to
-// different dies, each of which then keeps its heads' keys in its L2) and the tiles with the most keys come first.
+// different dies, each of which then keeps its heads' keys in its L2), the tiles in the order of the host's list
+// (which puts those with the most keys first).
 template <bool POW2>
 __global__ __launch_bounds__(256) void sigattn_prefill_kernel(
     const uint16_t* __restrict__ q, int q_stride, const uint16_t* __restrict__ k_pages,
@@ -231,7 +232,7 @@ __global__ __launch_bounds__(256) void sigattn_prefill_kernel(
     const float* __restrict__ r2, const float* __restrict__ pb, int nh, int nkv, int ps, int num_pages, float scale) {
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, j = lane & 15, qd = lane >> 4;
   const int lin = blockIdx.x;
-  const int tile = num_tiles - 1 - lin / nh, h = lin - (lin / nh) * nh;
+  const int tile = lin / nh, h = lin - tile * nh;
   const int sidx = tiles[2 * tile], row0 = tiles[2 * tile + 1];
   const int qstart = seq_starts[sidx], qlen = seq_starts[sidx + 1] - qstart, ctx = seq_ctx[sidx];
   const int rb = row0 + wave * 16;

@@ -1299,6 +1299,42 @@ def gla_scan(proj: torch.Tensor, q_col: int, k_col: int, v_col: int, z: torch.Te
     return out
 
 
+def gla_chunked(proj: torch.Tensor, q_col: int, k_col: int, v_col: int, z: torch.Tensor, z_bias: Optional[torch.Tensor],
+                tau: float, q_scale: float, state: torch.Tensor, out: torch.Tensor, seq_starts: torch.Tensor,
+                state_slots: torch.Tensor, tiles: torch.Tensor, num_tiles: int, first_request: int, nh: int, dim: int,
+                vdim: int, records: Optional[torch.Tensor] = None, decay: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """:func:`gla_scan` for the requests that ``tiles`` names (int32 [n, 2] of (request, first row of a tile of
+    PREFILL_TILE_ROWS among the request's rows) in any order: every tile of the requests from ``first_request`` on,
+    once): the tiles run side by side, first each
+    from a zero state, then a walk over every request's tiles leaves each the state before it, then each again from
+    that state, writing its rows; the last leaves the request's slot moved on.  ``records`` fp32 [>= n,
+    gla_state_floats] and ``decay`` fp32 [>= n, nh dim] are scratch."""
+    N = proj.shape[0]
+    _rows(proj, max(q_col + nh * dim, k_col + nh * dim, v_col + nh * vdim), "gla_chunked rows")
+    _need(z.is_cuda and z.dtype == torch.float32 and z.dim() == 2 and z.stride(1) == 1 and z.shape[1] >= nh * dim
+          and z.shape[0] == N, "gla_chunked: z fp32 [N, nh dim]")
+    _f32(z_bias, nh * dim, "gla_chunked bias")
+    _need(out.is_cuda and out.dtype == torch.float32 and out.is_contiguous() and tuple(out.shape) == (N, nh * vdim),
+          "gla_chunked: out [N, nh vdim] fp32")
+    _dev(seq_starts, state_slots, tiles)
+    _need(seq_starts.dtype == torch.int32 and state_slots.dtype == torch.int32 and tiles.dtype == torch.int32
+          and tiles.is_contiguous() and tiles.numel() >= 2 * num_tiles, "gla_chunked: int32 starts, slots and tiles")
+    floats = gla_state_floats(nh, dim, vdim)
+    stride = _state_rows(state, floats, "gla_chunked")
+    if records is None:
+        records = torch.empty((max(num_tiles, 1), floats), dtype=torch.float32, device=out.device)
+    if decay is None:
+        decay = torch.empty((max(num_tiles, 1), nh * dim), dtype=torch.float32, device=out.device)
+    _need(records.dtype == torch.float32 and records.is_contiguous() and records.numel() >= num_tiles * floats
+          and decay.dtype == torch.float32 and decay.is_contiguous() and decay.numel() >= num_tiles * nh * dim,
+          "gla_chunked: scratch for every tile")
+    _ok(_core().ia_gla_chunked(_p(proj), DTYPE_CODE[proj.dtype], int(proj.stride(0)), q_col, k_col, v_col, _p(z),
+                               int(z.stride(0)), _p(z_bias), ctypes.c_float(tau), ctypes.c_float(q_scale), _p(state),
+                               ctypes.c_long(stride), _p(out), _p(seq_starts), _p(state_slots), _p(tiles), int(num_tiles),
+                               int(first_request), _p(records), ctypes.c_long(floats), _p(decay), nh, dim, vdim, _stream()), "gla_chunked")
+    return out
+
+
 def head_norm_gate(o: torch.Tensor, gate: torch.Tensor, gate_col: int, w: torch.Tensor, eps: float, nh: int, vdim: int,
                    out: torch.Tensor) -> torch.Tensor:
     """out = o / sqrt(mean(o^2) + eps) * w * silu(gate) with the mean over each head's vdim values: o fp32 [N, nh vdim],

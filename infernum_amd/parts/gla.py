@@ -15,7 +15,7 @@ activations' type.
 """
 from __future__ import annotations
 
-from typing import Dict, Optional, Sequence
+from typing import Any, Dict, Optional, Sequence
 
 import torch
 
@@ -61,6 +61,10 @@ class GatedLinearAttention(Mixer):
                 a2b: WeightSpec((nq,), ("uniform", 1.0, 4.0), **small),
                 norm: WeightSpec((self.vdim,), ("uniform", 0.8, 1.2), **small), o: WeightSpec((H, nv), init)}
 
+    def step_needs(self) -> Dict[str, Any]:
+        # portions of prompts run as tiles of rows side by side
+        return {"row_tiles": K.PREFILL_TILE_ROWS}
+
     def load(self, tensors: Dict[str, torch.Tensor]) -> None:
         q, k, v, g, a1, a2, a2b, norm, o = self.names
         self.w_in = torch.cat([tensors[q], tensors[k], tensors[v], tensors[g]], dim=0).contiguous()
@@ -85,8 +89,14 @@ class GatedLinearAttention(Mixer):
         mid = linear(x, self.w_a1, kernels=self.rt.kernels)
         z = linear(mid, self.w_a2, out_dtype=torch.float32, kernels=self.rt.kernels)
         o = torch.empty((n, nv), dtype=torch.float32, device=dev)
-        K.gla_scan(proj, self.q_col, self.k_col, self.v_col, z, self.b_a2, self.tau, self.q_scale, state, o,
-                   ctx.seq_starts, ctx.state_slots, self.nh, self.dim, self.vdim)
+        nd = ctx.num_decode
+        if nd > 0:          # single tokens: the recurrence itself, a workgroup per request, head and slice of the state
+            K.gla_scan(proj, self.q_col, self.k_col, self.v_col, z, self.b_a2, self.tau, self.q_scale, state, o,
+                       ctx.seq_starts[:nd + 1], ctx.state_slots[:nd], self.nh, self.dim, self.vdim)
+        if ctx.num_seqs > nd:          # portions of prompts: tiles of rows side by side
+            tiles, num_tiles = ctx.row_tiles(K.PREFILL_TILE_ROWS)
+            K.gla_chunked(proj, self.q_col, self.k_col, self.v_col, z, self.b_a2, self.tau, self.q_scale, state, o,
+                          ctx.seq_starts, ctx.state_slots, tiles, num_tiles, nd, self.nh, self.dim, self.vdim)
         gated = torch.empty((n, nv), dtype=self.rt.dtype, device=dev)
         K.head_norm_gate(o, proj, self.g_col, self.w_norm, self.norm_eps, self.nh, self.vdim, gated)
         return linear(gated, self.w_o, keep_split=True, kernels=self.rt.kernels)
@@ -103,10 +113,22 @@ class GatedLinearAttention(Mixer):
         mid = emit_linear(program, program.x, N, self.w_a1, rt.dtype, None, False, "gla.mid", "gla.a1").tensor()
         z = emit_linear(program, mid, N, self.w_a2, torch.float32, None, False, "gla.z", "gla.a2").tensor()
         o = program.buffer("gla.o", T * nv * 4)
+        from ..engine.program import Guard
         program.op("core", "ia_gla_scan", [proj, act, self.row, self.q_col, self.k_col, self.v_col, z, nq, self.b_a2,
                                            float(self.tau), float(self.q_scale), state, int(state.stride(0)), o,
-                                           program.seq_starts, program.state_slots, program.B, self.nh, self.dim,
-                                           self.vdim, STREAM])
+                                           program.seq_starts, program.state_slots, program.ND, self.nh, self.dim,
+                                           self.vdim, STREAM], Guard.between(program.ND, 1))
+        # a request holds a state slot, and a tile at least one row: so many tiles a step has at most
+        floats = K.gla_state_floats(self.nh, self.dim, self.vdim)
+        most = -(-T // K.PREFILL_TILE_ROWS) + int(state.shape[0])
+        records = program.buffer("gla.records", most * floats * 4)
+        decay = program.buffer("gla.decay", most * nq * 4)
+        tiles, num_tiles = program.row_tiles(K.PREFILL_TILE_ROWS)
+        program.op("core", "ia_gla_chunked", [proj, act, self.row, self.q_col, self.k_col, self.v_col, z, nq, self.b_a2,
+                                              float(self.tau), float(self.q_scale), state, int(state.stride(0)), o,
+                                              program.seq_starts, program.state_slots, tiles, num_tiles, program.ND, records,
+                                              floats,
+                                              decay, self.nh, self.dim, self.vdim, STREAM], Guard.between(program.NP, 1))
         gated = program.buffer("gla.gated", T * nv * ab)
         program.op("core", "ia_head_norm_gate", [o, proj, act, self.row, self.g_col, self.w_norm, gated, N, self.nh,
                                                  self.vdim, float(self.norm_eps), STREAM])
