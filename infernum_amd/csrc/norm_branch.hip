@@ -227,18 +227,134 @@ __global__ __launch_bounds__(NB_NT) void gated_norm_add_kernel(float* __restrict
     x[(size_t)row * H + i] = from_float<TX>(w_next ? hr[i] * inv2 * load_as_float(w_next, w_next_dtype, i) : hr[i]);
 }
 
+// The same for rows of a multiple of 4 values up to NT * 4 * NV, with every pointer and stride a multiple of 16 bytes:
+// a thread keeps its pieces of the row in registers, read 16 (or 8) bytes at a time, the loads of all parts of a piece
+// in flight together; one pass over memory.  The sums of a row are taken in one order whatever the batch holds.
+__device__ __forceinline__ float4 nb_load4_any(const void* p, int dtype, int i) {
+  return dtype == IA_F32 ? nb_load4((const float*)p + i) : nb_load4((const bf16_t*)p + i);
+}
+
+template <typename TD, typename TG, typename TX, int NT, int NV>
+__global__ __launch_bounds__(NT) void gated_norm_add_vec_kernel(float* __restrict__ h, const TD* __restrict__ delta,
+                                                                int splits, size_t split_stride,
+                                                                const TG* __restrict__ gate, int gate_stride,
+                                                                const float* __restrict__ gate_bias,
+                                                                const void* __restrict__ w, int w_dtype,
+                                                                const void* __restrict__ w_next, int w_next_dtype,
+                                                                TX* __restrict__ x, int H, float eps) {
+  __shared__ float red[NT / 64];
+  const int row = blockIdx.x;
+  const TD* dr = delta + (size_t)row * H;
+  float* hr = h + (size_t)row * H;
+  float4 d[NV], hv[NV];
+#pragma unroll
+  for (int c = 0; c < NV; ++c) {
+    const int i = (threadIdx.x + c * NT) * 4;
+    d[c] = hv[c] = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (i < H) {
+      hv[c] = nb_load4(hr + i);
+      d[c] = nb_load4(dr + i);
+    }
+  }
+#pragma clang loop unroll_count(4)
+  for (int k = 1; k < splits; ++k) {                 // the parts in the order of their index
+#pragma unroll
+    for (int c = 0; c < NV; ++c) {
+      const int i = (threadIdx.x + c * NT) * 4;
+      if (i < H) {
+        const float4 p = nb_load4(dr + k * split_stride + i);
+        d[c].x += p.x; d[c].y += p.y; d[c].z += p.z; d[c].w += p.w;
+      }
+    }
+  }
+  if (gate) {
+#pragma unroll
+    for (int c = 0; c < NV; ++c) {
+      const int i = (threadIdx.x + c * NT) * 4;
+      if (i < H) {
+        float4 z = nb_load4(gate + (size_t)row * gate_stride + i);
+        if (gate_bias) {
+          const float4 b = nb_load4(gate_bias + i);
+          z.x += b.x; z.y += b.y; z.z += b.z; z.w += b.w;
+        }
+        d[c].x *= 1.0f / (1.0f + expf(-z.x));
+        d[c].y *= 1.0f / (1.0f + expf(-z.y));
+        d[c].z *= 1.0f / (1.0f + expf(-z.z));
+        d[c].w *= 1.0f / (1.0f + expf(-z.w));
+      }
+    }
+  }
+  float ss = 0.f;
+#pragma unroll
+  for (int c = 0; c < NV; ++c)
+    ss += __builtin_fmaf(d[c].x, d[c].x, d[c].y * d[c].y) + __builtin_fmaf(d[c].z, d[c].z, d[c].w * d[c].w);
+  ss = block_sum<NT>(ss, red);
+  const float inv = 1.0f / sqrtf(ss / (float)H + eps);
+  float s2 = 0.f;
+#pragma unroll
+  for (int c = 0; c < NV; ++c) {
+    const int i = (threadIdx.x + c * NT) * 4;
+    if (i < H) {
+      const float4 g = nb_load4_any(w, w_dtype, i);
+      hv[c] = make_float4(hv[c].x + d[c].x * inv * g.x, hv[c].y + d[c].y * inv * g.y, hv[c].z + d[c].z * inv * g.z,
+                          hv[c].w + d[c].w * inv * g.w);
+      nb_store4(hr + i, hv[c]);
+      s2 += __builtin_fmaf(hv[c].x, hv[c].x, hv[c].y * hv[c].y) + __builtin_fmaf(hv[c].z, hv[c].z, hv[c].w * hv[c].w);
+    }
+  }
+  if (!x) return;
+  float inv2 = 1.0f;
+  if (w_next) {
+    s2 = block_sum<NT>(s2, red);
+    inv2 = 1.0f / sqrtf(s2 / (float)H + eps);
+  }
+#pragma unroll
+  for (int c = 0; c < NV; ++c) {
+    const int i = (threadIdx.x + c * NT) * 4;
+    if (i < H) {
+      float4 o = hv[c];
+      if (w_next) {
+        const float4 g = nb_load4_any(w_next, w_next_dtype, i);
+        o = make_float4(o.x * inv2 * g.x, o.y * inv2 * g.y, o.z * inv2 * g.z, o.w * inv2 * g.w);
+      }
+      nb_store4(x + (size_t)row * H + i, o);
+    }
+  }
+}
+
+template <typename TD, typename TG, typename TX>
+static void launch_gated_norm_add_typed(float* h, const TD* delta, int splits, size_t stride, const TG* gate,
+                                        int gate_stride, const float* gate_bias, const void* w, int w_dtype,
+                                        const void* w_next, int w_next_dtype, TX* x, int N, int H, float eps,
+                                        hipStream_t stream) {
+  const bool aligned = ((reinterpret_cast<uintptr_t>(h) | reinterpret_cast<uintptr_t>(delta) |
+                         reinterpret_cast<uintptr_t>(gate) | reinterpret_cast<uintptr_t>(gate_bias) |
+                         reinterpret_cast<uintptr_t>(w) | reinterpret_cast<uintptr_t>(w_next) |
+                         reinterpret_cast<uintptr_t>(x)) & 15) == 0 &&
+                       (stride & 3) == 0 && (gate_stride & 3) == 0 && (H & 3) == 0;
+#define IA_GNA_VEC(NT, NV)                                                                                          \
+  gated_norm_add_vec_kernel<TD, TG, TX, NT, NV><<<N, NT, 0, stream>>>(h, delta, splits, stride, gate, gate_stride,  \
+                                                                      gate_bias, w, w_dtype, w_next, w_next_dtype, x, \
+                                                                      H, eps)
+  if (aligned && H <= 256 * 4) IA_GNA_VEC(256, 1);           // the kernel follows from H alone: a row's sums are taken
+  else if (aligned && H <= 1024 * 4) IA_GNA_VEC(1024, 1);    // in one order
+  else if (aligned && H <= 1024 * 4 * 4) IA_GNA_VEC(1024, 4);
+  else
+    gated_norm_add_kernel<TD, TG, TX><<<N, NB_NT, 0, stream>>>(h, delta, splits, stride, gate, gate_stride, gate_bias, w,
+                                                               w_dtype, w_next, w_next_dtype, x, H, eps);
+#undef IA_GNA_VEC
+}
+
 template <typename TD, typename TX>
 static int launch_gated_norm_add(float* h, const void* delta, int splits, size_t stride, const void* gate, int gate_dtype,
                                  int gate_stride, const float* gate_bias, const void* w, int w_dtype, const void* w_next,
                                  int w_next_dtype, void* x, int N, int H, float eps, hipStream_t stream) {
   if (gate_dtype == IA_F32)
-    gated_norm_add_kernel<TD, float, TX><<<N, NB_NT, 0, stream>>>(h, (const TD*)delta, splits, stride, (const float*)gate,
-                                                                  gate_stride, gate_bias, w, w_dtype, w_next, w_next_dtype,
-                                                                  (TX*)x, H, eps);
+    launch_gated_norm_add_typed<TD, float, TX>(h, (const TD*)delta, splits, stride, (const float*)gate, gate_stride,
+                                               gate_bias, w, w_dtype, w_next, w_next_dtype, (TX*)x, N, H, eps, stream);
   else if (gate_dtype == IA_BF16)
-    gated_norm_add_kernel<TD, bf16_t, TX><<<N, NB_NT, 0, stream>>>(h, (const TD*)delta, splits, stride, (const bf16_t*)gate,
-                                                                   gate_stride, gate_bias, w, w_dtype, w_next, w_next_dtype,
-                                                                   (TX*)x, H, eps);
+    launch_gated_norm_add_typed<TD, bf16_t, TX>(h, (const TD*)delta, splits, stride, (const bf16_t*)gate, gate_stride,
+                                                gate_bias, w, w_dtype, w_next, w_next_dtype, (TX*)x, N, H, eps, stream);
   else
     return IA_ERR_BAD_ARG;
   return IA_OK;

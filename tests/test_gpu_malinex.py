@@ -91,7 +91,7 @@ def test_learned_position_rows(dtype):
 
 
 @BOTH
-@pytest.mark.parametrize("N,H,splits", [(1, 64, 0), (9, 100, 0), (70, 256, 3), (5, 48, 2), (300, 2048, 0)])
+@pytest.mark.parametrize("N,H,splits", [(1, 64, 0), (9, 100, 0), (70, 256, 3), (5, 48, 2), (300, 2048, 0), (3, 4100, 2), (4, 6, 0), (2, 16388, 0)])
 @pytest.mark.parametrize("gated,nxt", [(True, True), (True, False), (False, True)])
 def test_gated_branch_norm(dtype, N, H, splits, gated, nxt):
     """h += norm(delta * sigmoid(G + b)) and, with a next norm, its rows besides; the delta a tensor or partial sums."""
