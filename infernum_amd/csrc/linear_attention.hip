@@ -141,8 +141,10 @@ __global__ __launch_bounds__(256) void gla_scan_kernel(
   }
 }
 
-// grid (heads x slices, tiles), 256 threads; the workgroup of a request's first tile walks the request's tiles: the
-// record of a tile holds what the tile adds when it comes and the state before the tile when it goes.
+// grid (heads x slices x blocks of 256 values, tiles), 256 threads, a value of the state a thread; the workgroups of
+// a request's first tile walk the request's tiles: the record of a tile holds what the tile adds when they come and
+// the state before the tile when they go.  Eight tiles' loads are in flight together.
+#define GLA_CHAIN_AHEAD 8
 __global__ __launch_bounds__(256) void gla_chain_kernel(const float* __restrict__ state, long state_stride,
                                                         const int* __restrict__ seq_starts,
                                                         const int* __restrict__ state_slots, const int* __restrict__ tiles,
@@ -151,20 +153,30 @@ __global__ __launch_bounds__(256) void gla_chain_kernel(const float* __restrict_
   const int i = blockIdx.y;
   if (tiles[2 * i + 1] != 0) return;
   const int s = tiles[2 * i], rows = seq_starts[s + 1] - seq_starts[s];
-  const int hs = blockIdx.x, hd = hs / slices;
-  const size_t within = (size_t)hs * dim * GLA_PW;
-  const float* S0 = state + (size_t)state_slots[s] * state_stride + within;
+  const int per = (dim * GLA_PW + 255) / 256;
+  const int hs = blockIdx.x / per, e = (blockIdx.x - hs * per) * 256 + threadIdx.x;
+  if (e >= dim * GLA_PW) return;
+  const int hd = hs / slices, n = e / GLA_PW;
+  const size_t within = (size_t)hs * dim * GLA_PW + e;
   const int first = gla_record(seq_starts, first_request, s, 0);
-  for (int e = threadIdx.x; e < dim * GLA_PW; e += 256) {
-    const int n = e / GLA_PW;
-    float S = S0[e];
-    int j = first;
-    for (int r0 = 0; r0 < rows; r0 += GLA_TILE, ++j) {
-      float* at = records + (size_t)j * record_stride + within + e;
-      const bool last = r0 + GLA_TILE >= rows;
-      const float U = last ? 0.f : *at;
-      *at = S;
-      if (!last) S = __builtin_fmaf(decay[((size_t)j * nh + hd) * dim + n], S, U);
+  const int count = (rows + GLA_TILE - 1) / GLA_TILE;
+  float S = state[(size_t)state_slots[s] * state_stride + within];
+  for (int j0 = 0; j0 < count; j0 += GLA_CHAIN_AHEAD) {
+    float U[GLA_CHAIN_AHEAD], D[GLA_CHAIN_AHEAD];
+#pragma unroll
+    for (int a = 0; a < GLA_CHAIN_AHEAD; ++a) {
+      const int j = j0 + a;
+      const bool adds = j < count - 1;                       // a request's last tile adds nothing that anyone reads
+      U[a] = adds ? records[(size_t)(first + j) * record_stride + within] : 0.f;
+      D[a] = adds ? decay[((size_t)(first + j) * nh + hd) * dim + n] : 0.f;
+    }
+#pragma unroll
+    for (int a = 0; a < GLA_CHAIN_AHEAD; ++a) {
+      const int j = j0 + a;
+      if (j < count) {
+        records[(size_t)(first + j) * record_stride + within] = S;
+        if (j < count - 1) S = __builtin_fmaf(D[a], S, U[a]);
+      }
     }
   }
 }
@@ -251,7 +263,7 @@ extern "C" int ia_gla_chunked(const void* proj, int code, int proj_stride, int q
   if (code != IA_F32 && code != IA_BF16) return IA_ERR_BAD_ARG;
   IA_GLA_T(1);
   IA_LAUNCH_CHECK();
-  gla_chain_kernel<<<dim3((unsigned)(nh * slices), (unsigned)num_tiles), 256, 0, stream>>>(
+  gla_chain_kernel<<<dim3((unsigned)(nh * slices * ((dim * GLA_PW + 255) / 256)), (unsigned)num_tiles), 256, 0, stream>>>(
       state, state_stride, seq_starts, state_slots, tiles, first_request, records, record_stride, decay, nh, dim, slices);
   IA_LAUNCH_CHECK();
   IA_GLA_T(2);
