@@ -52,8 +52,7 @@ class SigmoidAttention(Mixer):
         if kernels not in ("auto", "generic"):
             raise ValueError("kernels must be 'auto' or 'generic'")
         self.use_mfma = (kernels == "auto" and rt.kernels == "auto" and rt.dtype == torch.bfloat16
-                         and rt.device.type == "cuda" and K.sigattn_mfma_available(self.dim, self.vdim)
-                         and self.nq % 8 == 0 and self.row % 8 == 0)
+                         and rt.device.type == "cuda" and K.sigattn_mfma_available(self.dim, self.vdim))
 
     # ---- what it needs ---------------------------------------------------
     def cache_spec(self) -> CacheSpec:
