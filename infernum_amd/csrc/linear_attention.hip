@@ -49,7 +49,7 @@ __global__ __launch_bounds__(256) void gla_scan_kernel(
     long state_stride, float* __restrict__ out, const int* __restrict__ seq_starts, const int* __restrict__ state_slots,
     int nh, int dim, int vdim, const int* __restrict__ tiles, int first_request, float* __restrict__ records,
     long record_stride, float* __restrict__ decay) {
-  extern __shared__ float lds[];
+  extern __shared__ __attribute__((aligned(16))) float lds[];
   float* qs = lds;                                   // [TB][dim]
   float* ks = qs + GLA_TB * dim;                     // [TB][dim]
   float* as = ks + GLA_TB * dim;                     // [TB][dim]  alpha
@@ -70,6 +70,7 @@ __global__ __launch_bounds__(256) void gla_scan_kernel(
   }
   if (count <= 0) return;
   const int tid = threadIdx.x;
+  const bool vec = (dim & 3) == 0;
   const int p = tid % GLA_PW, part = tid / GLA_PW;
   const int col = slice * GLA_PW + p;
   const int slices = gla_slices(vdim);
@@ -80,7 +81,7 @@ __global__ __launch_bounds__(256) void gla_scan_kernel(
   float reg[KMAX];
 #pragma unroll
   for (int c = 0; c < KMAX; ++c) {
-    const int n = part + c * GLA_PARTS;
+    const int n = part * KMAX + c;
     reg[c] = (MODE != 1 && n < dim) ? R[(size_t)n * GLA_PW + p] : 0.f;
     if constexpr (MODE == 1) dprod[c] = 1.f;
   }
@@ -93,8 +94,9 @@ __global__ __launch_bounds__(256) void gla_scan_kernel(
       const T* pr = proj + row * proj_stride;
       qs[i] = to_float(pr[q_col + hd * dim + n]) * q_scale;
       ks[i] = to_float(pr[k_col + hd * dim + n]);
-      const float zz = z[row * z_stride + hd * dim + n] + (z_bias ? z_bias[hd * dim + n] : 0.f);
-      as[i] = expf(gla_log_sigmoid(zz) * inv_tau);
+      const float zz = z[row * z_stride + hd * dim + n];
+      // the tiles read decays that one kernel made of the logits before them; the walk over a request makes its own
+      as[i] = MODE != 0 ? zz : expf(gla_log_sigmoid(zz + (z_bias ? z_bias[hd * dim + n] : 0.f)) * inv_tau);
     }
     for (int i = tid; i < nt * GLA_PW; i += 256) {
       const int t = i / GLA_PW, c = slice * GLA_PW + (i - t * GLA_PW);
@@ -108,12 +110,34 @@ __global__ __launch_bounds__(256) void gla_scan_kernel(
       const float* at = as + t * dim;
       float acc = 0.f;
 #pragma unroll
-      for (int c = 0; c < KMAX; ++c) {
-        const int n = part + c * GLA_PARTS;
-        if (n < dim) {
-          reg[c] = __builtin_fmaf(at[n], reg[c], kt[n] * v);
-          if constexpr (MODE == 1) dprod[c] *= at[n];
-          else acc = __builtin_fmaf(reg[c], qt[n], acc);
+      for (int c4 = 0; c4 < KMAX; c4 += 4) {          // a thread's channels lie side by side: 16 bytes a read
+        const int n0 = part * KMAX + c4;
+        float a4[4], k4[4], q4[4];
+        if (vec) {
+          const bool in = n0 < dim;
+          const float4 av = in ? *reinterpret_cast<const float4*>(at + n0) : make_float4(0.f, 0.f, 0.f, 0.f);
+          const float4 kv = in ? *reinterpret_cast<const float4*>(kt + n0) : make_float4(0.f, 0.f, 0.f, 0.f);
+          a4[0] = av.x; a4[1] = av.y; a4[2] = av.z; a4[3] = av.w;
+          k4[0] = kv.x; k4[1] = kv.y; k4[2] = kv.z; k4[3] = kv.w;
+          if (MODE != 1) {
+            const float4 qv = in ? *reinterpret_cast<const float4*>(qt + n0) : make_float4(0.f, 0.f, 0.f, 0.f);
+            q4[0] = qv.x; q4[1] = qv.y; q4[2] = qv.z; q4[3] = qv.w;
+          }
+        } else {
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const bool in = n0 + e < dim;
+            a4[e] = in ? at[n0 + e] : 0.f;
+            k4[e] = in ? kt[n0 + e] : 0.f;
+            q4[e] = (MODE != 1 && in) ? qt[n0 + e] : 0.f;
+          }
+        }
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {                  // channels past the head's last stay zero: 0 * 0 + 0 * v
+          const int c = c4 + e;
+          reg[c] = __builtin_fmaf(a4[e], reg[c], k4[e] * v);
+          if constexpr (MODE == 1) dprod[c] *= a4[e];
+          else acc = __builtin_fmaf(reg[c], q4[e], acc);
         }
       }
       if (MODE != 1) ysum[(t * GLA_PARTS + part) * GLA_PW + p] = acc;
@@ -133,7 +157,7 @@ __global__ __launch_bounds__(256) void gla_scan_kernel(
   float* W = MODE == 1 ? R : S;
 #pragma unroll
   for (int c = 0; c < KMAX; ++c) {
-    const int n = part + c * GLA_PARTS;
+    const int n = part * KMAX + c;
     if (n < dim) {
       W[(size_t)n * GLA_PW + p] = reg[c];
       if constexpr (MODE == 1) if (p == 0 && slice == 0) decay[((size_t)record * nh + hd) * dim + n] = dprod[c];
@@ -223,16 +247,31 @@ extern "C" int ia_gla_scan(const void* proj, int code, int proj_stride, int q_co
   return IA_OK;
 }
 
+// z <- alpha = exp(log_sigmoid(z + bias) / tau) in place, for the rows from request ``first_request``'s first on.
+__global__ __launch_bounds__(256) void gla_decays_kernel(float* __restrict__ z, int z_stride, const float* __restrict__ z_bias,
+                                                         float inv_tau, const int* __restrict__ seq_starts,
+                                                         int first_request, int num_rows, int cols) {
+  const int row0 = seq_starts[first_request];
+  const size_t total = (size_t)(num_rows - row0) * cols, stride = (size_t)gridDim.x * 256;
+  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < total; i += stride) {
+    const size_t r = i / cols;
+    const int c = (int)(i - r * cols);
+    float* at = z + (row0 + r) * z_stride + c;
+    *at = expf(gla_log_sigmoid(*at + (z_bias ? z_bias[c] : 0.f)) * inv_tau);
+  }
+}
+
 // The recurrence of ia_gla_scan for the requests that the tiles name: tiles[i] = (request, first row of a tile of
 // GLA_TILE among the request's rows) in any order, every tile of the requests first_request .. (and of no other)
-// once.  records: fp32 [num_tiles, record_stride >= ia_gla_state_floats]; decay: fp32 [num_tiles, nh, dim].
+// once.  records: fp32 [num_tiles, record_stride >= ia_gla_state_floats]; decay: fp32 [num_tiles, nh, dim].  z has
+// num_rows rows; those of the requests first_request .. are left holding the decays, not the logits.
 extern "C" int ia_gla_chunked(const void* proj, int code, int proj_stride, int q_col, int k_col, int v_col, const float* z,
                               int z_stride, const float* z_bias, float tau, float q_scale, float* state,
                               long state_stride, float* out, const int* seq_starts, const int* state_slots,
-                              const int* tiles, int num_tiles, int first_request, float* records, long record_stride, float* decay, int nh,
+                              const int* tiles, int num_tiles, int first_request, int num_rows, float* records, long record_stride, float* decay, int nh,
                               int dim, int vdim, hipStream_t stream) {
   if (num_tiles == 0) return IA_OK;
-  if (!proj || !z || !state || !out || !seq_starts || !state_slots || !tiles || !records || !decay || num_tiles < 0 || first_request < 0 ||
+  if (!proj || !z || !state || !out || !seq_starts || !state_slots || !tiles || !records || !decay || num_tiles < 0 || first_request < 0 || num_rows <= 0 ||
       nh <= 0 || dim <= 0 || vdim <= 0 || !(tau > 0.f) || q_col < 0 || k_col < 0 || v_col < 0 ||
       proj_stride < q_col + nh * dim || proj_stride < k_col + nh * dim || proj_stride < v_col + nh * vdim ||
       z_stride < nh * dim || state_stride < ia_gla_state_floats(nh, dim, vdim) ||
@@ -261,6 +300,12 @@ extern "C" int ia_gla_chunked(const void* proj, int code, int proj_stride, int q
     else IA_GLA_K(bf16_t, MODE);                   \
   } while (0)
   if (code != IA_F32 && code != IA_BF16) return IA_ERR_BAD_ARG;
+  {
+    const size_t most = (size_t)num_rows * nh * dim;
+    gla_decays_kernel<<<(unsigned)((most + 255) / 256 < 262144 ? (most + 255) / 256 : 262144), 256, 0, stream>>>(
+        const_cast<float*>(z), z_stride, z_bias, 1.0f / tau, seq_starts, first_request, num_rows, nh * dim);
+    IA_LAUNCH_CHECK();
+  }
   IA_GLA_T(1);
   IA_LAUNCH_CHECK();
   gla_chain_kernel<<<dim3((unsigned)(nh * slices * ((dim * GLA_PW + 255) / 256)), (unsigned)num_tiles), 256, 0, stream>>>(

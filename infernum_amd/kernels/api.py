@@ -1308,7 +1308,8 @@ def gla_chunked(proj: torch.Tensor, q_col: int, k_col: int, v_col: int, z: torch
     once): the tiles run side by side, first each
     from a zero state, then a walk over every request's tiles leaves each the state before it, then each again from
     that state, writing its rows; the last leaves the request's slot moved on.  ``records`` fp32 [>= n,
-    gla_state_floats] and ``decay`` fp32 [>= n, nh dim] are scratch."""
+    gla_state_floats] and ``decay`` fp32 [>= n, nh dim] are scratch.  The rows of ``z`` that belong to those requests are left
+    holding the decays, not the logits."""
     N = proj.shape[0]
     _rows(proj, max(q_col + nh * dim, k_col + nh * dim, v_col + nh * vdim), "gla_chunked rows")
     _need(z.is_cuda and z.dtype == torch.float32 and z.dim() == 2 and z.stride(1) == 1 and z.shape[1] >= nh * dim
@@ -1331,7 +1332,7 @@ def gla_chunked(proj: torch.Tensor, q_col: int, k_col: int, v_col: int, z: torch
     _ok(_core().ia_gla_chunked(_p(proj), DTYPE_CODE[proj.dtype], int(proj.stride(0)), q_col, k_col, v_col, _p(z),
                                int(z.stride(0)), _p(z_bias), ctypes.c_float(tau), ctypes.c_float(q_scale), _p(state),
                                ctypes.c_long(stride), _p(out), _p(seq_starts), _p(state_slots), _p(tiles), int(num_tiles),
-                               int(first_request), _p(records), ctypes.c_long(floats), _p(decay), nh, dim, vdim, _stream()), "gla_chunked")
+                               int(first_request), int(N), _p(records), ctypes.c_long(floats), _p(decay), nh, dim, vdim, _stream()), "gla_chunked")
     return out
 
 

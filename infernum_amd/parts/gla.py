@@ -126,7 +126,7 @@ class GatedLinearAttention(Mixer):
         tiles, num_tiles = program.row_tiles(K.PREFILL_TILE_ROWS)
         program.op("core", "ia_gla_chunked", [proj, act, self.row, self.q_col, self.k_col, self.v_col, z, nq, self.b_a2,
                                               float(self.tau), float(self.q_scale), state, int(state.stride(0)), o,
-                                              program.seq_starts, program.state_slots, tiles, num_tiles, program.ND, records,
+                                              program.seq_starts, program.state_slots, tiles, num_tiles, program.ND, N, records,
                                               floats,
                                               decay, self.nh, self.dim, self.vdim, STREAM], Guard.between(program.NP, 1))
         gated = program.buffer("gla.gated", T * nv * ab)
