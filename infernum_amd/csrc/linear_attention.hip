@@ -6,7 +6,8 @@
 //
 //   ia_gla_scan         the recurrence token after token for the rows of every request of a step, from the request's
 //                       state slot, which it leaves moved on;
-//   ia_gla_chunked      the same for portions of prompts cut into tiles of GLA_TILE rows that run side by side: every
+//   ia_gla_chunked      the same for portions of prompts cut into tiles of GLA_TILE rows that run side by side, behind
+//                       a kernel that turns the portions' decay logits into decays once, in place: every
 //                       tile but a request's last first runs from a zero state and leaves what it adds, U, and the
 //                       product D of its decays; a second kernel walks a request's tiles, S <- diag(D) S + U, and
 //                       leaves every tile the state before it; then every tile runs from that state and writes its
