@@ -163,6 +163,7 @@ template <typename TD, typename TG, typename TX>
 __global__ __launch_bounds__(NB_NT) void gated_norm_add_kernel(float* __restrict__ h, const TD* __restrict__ delta,
                                                                int splits, size_t split_stride,
                                                                const TG* __restrict__ gate, int gate_stride,
+                                                               int gate_splits, size_t gate_split_stride,
                                                                const float* __restrict__ gate_bias,
                                                                const void* __restrict__ w, int w_dtype,
                                                                const void* __restrict__ w_next, int w_next_dtype,
@@ -175,7 +176,7 @@ __global__ __launch_bounds__(NB_NT) void gated_norm_add_kernel(float* __restrict
   auto gated = [&](int i) {
     float d = load_split_sum(dr + i, splits, split_stride);
     if (gr) {
-      const float z = to_float(gr[i]) + (gate_bias ? gate_bias[i] : 0.f);
+      const float z = load_split_sum(gr + i, gate_splits, gate_split_stride) + (gate_bias ? gate_bias[i] : 0.f);
       d *= 1.0f / (1.0f + expf(-z));
     }
     return d;
@@ -238,6 +239,7 @@ template <typename TD, typename TG, typename TX, int NT, int NV>
 __global__ __launch_bounds__(NT) void gated_norm_add_vec_kernel(float* __restrict__ h, const TD* __restrict__ delta,
                                                                 int splits, size_t split_stride,
                                                                 const TG* __restrict__ gate, int gate_stride,
+                                                                int gate_splits, size_t gate_split_stride,
                                                                 const float* __restrict__ gate_bias,
                                                                 const void* __restrict__ w, int w_dtype,
                                                                 const void* __restrict__ w_next, int w_next_dtype,
@@ -273,6 +275,10 @@ __global__ __launch_bounds__(NT) void gated_norm_add_vec_kernel(float* __restric
       const int i = (threadIdx.x + c * NT) * 4;
       if (i < H) {
         float4 z = nb_load4(gate + (size_t)row * gate_stride + i);
+        for (int k = 1; k < gate_splits; ++k) {        // the logits' parts in the order of their index
+          const float4 q = nb_load4(gate + k * gate_split_stride + (size_t)row * gate_stride + i);
+          z.x += q.x; z.y += q.y; z.z += q.z; z.w += q.w;
+        }
         if (gate_bias) {
           const float4 b = nb_load4(gate_bias + i);
           z.x += b.x; z.y += b.y; z.z += b.z; z.w += b.w;
@@ -324,61 +330,66 @@ __global__ __launch_bounds__(NT) void gated_norm_add_vec_kernel(float* __restric
 
 template <typename TD, typename TG, typename TX>
 static void launch_gated_norm_add_typed(float* h, const TD* delta, int splits, size_t stride, const TG* gate,
-                                        int gate_stride, const float* gate_bias, const void* w, int w_dtype,
+                                        int gate_stride, int gate_splits, size_t gate_split_stride, const float* gate_bias, const void* w, int w_dtype,
                                         const void* w_next, int w_next_dtype, TX* x, int N, int H, float eps,
                                         hipStream_t stream) {
   const bool aligned = ((reinterpret_cast<uintptr_t>(h) | reinterpret_cast<uintptr_t>(delta) |
                          reinterpret_cast<uintptr_t>(gate) | reinterpret_cast<uintptr_t>(gate_bias) |
                          reinterpret_cast<uintptr_t>(w) | reinterpret_cast<uintptr_t>(w_next) |
                          reinterpret_cast<uintptr_t>(x)) & 15) == 0 &&
-                       (stride & 3) == 0 && (gate_stride & 3) == 0 && (H & 3) == 0;
+                       (stride & 3) == 0 && (gate_stride & 3) == 0 && (gate_split_stride & 3) == 0 && (H & 3) == 0;
 #define IA_GNA_VEC(NT, NV)                                                                                          \
-  gated_norm_add_vec_kernel<TD, TG, TX, NT, NV><<<N, NT, 0, stream>>>(h, delta, splits, stride, gate, gate_stride,  \
-                                                                      gate_bias, w, w_dtype, w_next, w_next_dtype, x, \
-                                                                      H, eps)
+  gated_norm_add_vec_kernel<TD, TG, TX, NT, NV><<<N, NT, 0, stream>>>(                                             \
+      h, delta, splits, stride, gate, gate_stride, gate_splits, gate_split_stride, gate_bias, w, w_dtype, w_next,   \
+      w_next_dtype, x, H, eps)
   if (aligned && H <= 256 * 4) IA_GNA_VEC(256, 1);           // the kernel follows from H alone: a row's sums are taken
   else if (aligned && H <= 1024 * 4) IA_GNA_VEC(1024, 1);    // in one order
   else if (aligned && H <= 1024 * 4 * 4) IA_GNA_VEC(1024, 4);
   else
-    gated_norm_add_kernel<TD, TG, TX><<<N, NB_NT, 0, stream>>>(h, delta, splits, stride, gate, gate_stride, gate_bias, w,
-                                                               w_dtype, w_next, w_next_dtype, x, H, eps);
+    gated_norm_add_kernel<TD, TG, TX><<<N, NB_NT, 0, stream>>>(h, delta, splits, stride, gate, gate_stride, gate_splits,
+                                                               gate_split_stride, gate_bias, w, w_dtype, w_next,
+                                                               w_next_dtype, x, H, eps);
 #undef IA_GNA_VEC
 }
 
 template <typename TD, typename TX>
 static int launch_gated_norm_add(float* h, const void* delta, int splits, size_t stride, const void* gate, int gate_dtype,
-                                 int gate_stride, const float* gate_bias, const void* w, int w_dtype, const void* w_next,
+                                 int gate_stride, int gate_splits, size_t gate_split_stride, const float* gate_bias, const void* w, int w_dtype, const void* w_next,
                                  int w_next_dtype, void* x, int N, int H, float eps, hipStream_t stream) {
   if (gate_dtype == IA_F32)
     launch_gated_norm_add_typed<TD, float, TX>(h, (const TD*)delta, splits, stride, (const float*)gate, gate_stride,
-                                               gate_bias, w, w_dtype, w_next, w_next_dtype, (TX*)x, N, H, eps, stream);
+                                               gate_splits, gate_split_stride, gate_bias, w, w_dtype, w_next, w_next_dtype, (TX*)x, N, H, eps, stream);
   else if (gate_dtype == IA_BF16)
     launch_gated_norm_add_typed<TD, bf16_t, TX>(h, (const TD*)delta, splits, stride, (const bf16_t*)gate, gate_stride,
-                                                gate_bias, w, w_dtype, w_next, w_next_dtype, (TX*)x, N, H, eps, stream);
+                                                gate_splits, gate_split_stride, gate_bias, w, w_dtype, w_next, w_next_dtype, (TX*)x, N, H, eps, stream);
   else
     return IA_ERR_BAD_ARG;
   return IA_OK;
 }
 
-// delta [splits, delta_rows, H] of delta_dtype; gate (nullable) [N, >= H] rows of gate_stride values of gate_dtype;
+// delta [splits, delta_rows, H] of delta_dtype; gate (nullable) [gate_splits, gate_rows, >= H] rows of gate_stride
+// values of gate_dtype (parts of the logits, added in the order of their index; more than one part: fp32);
 // gate_bias (nullable) fp32 [H]; w_next (nullable): the weight of the norm that follows the add; x (nullable) of act_dtype.
 extern "C" int ia_gated_norm_add(float* h, const void* delta, int delta_dtype, int splits, int delta_rows, const void* gate,
-                                 int gate_dtype, int gate_stride, const float* gate_bias, const void* w, int w_dtype,
+                                 int gate_dtype, int gate_stride, int gate_splits, int gate_rows, const float* gate_bias, const void* w, int w_dtype,
                                  const void* w_next, int w_next_dtype, void* x, int act_dtype, int N, int H, float eps,
                                  hipStream_t stream) {
-  if (N < 0 || H <= 0 || !(eps > 0.f) || !delta || !h || !w || splits < 1 || delta_rows < N || (gate && gate_stride < H))
+  if (N < 0 || H <= 0 || !(eps > 0.f) || !delta || !h || !w || splits < 1 || delta_rows < N ||
+      (gate && (gate_stride < H || gate_splits < 1 || gate_rows < N || (gate_splits > 1 && gate_dtype != IA_F32))))
     return IA_ERR_BAD_ARG;
   if (N == 0) return IA_OK;
   const size_t stride = (size_t)delta_rows * H;
+  const size_t gstride = gate ? (size_t)gate_rows * gate_stride : 0;
+  if (!gate) gate_splits = 1;
   int rc;
   if (delta_dtype == IA_F32 && act_dtype == IA_F32)
-    rc = launch_gated_norm_add<float, float>(h, delta, splits, stride, gate, gate_dtype, gate_stride, gate_bias, w, w_dtype,
+    rc = launch_gated_norm_add<float, float>(h, delta, splits, stride, gate, gate_dtype, gate_stride, gate_splits, gstride, gate_bias, w, w_dtype,
                                              w_next, w_next_dtype, x, N, H, eps, stream);
   else if (delta_dtype == IA_BF16 && act_dtype == IA_BF16)
-    rc = launch_gated_norm_add<bf16_t, bf16_t>(h, delta, splits, stride, gate, gate_dtype, gate_stride, gate_bias, w,
+    rc = launch_gated_norm_add<bf16_t, bf16_t>(h, delta, splits, stride, gate, gate_dtype, gate_stride, gate_splits, gstride, gate_bias, w,
                                                w_dtype, w_next, w_next_dtype, x, N, H, eps, stream);
   else if (delta_dtype == IA_F32 && act_dtype == IA_BF16)
-    rc = launch_gated_norm_add<float, bf16_t>(h, delta, splits, stride, gate, gate_dtype, gate_stride, gate_bias, w,
+    rc = launch_gated_norm_add<float, bf16_t>(h, delta, splits, stride, gate, gate_dtype, gate_stride, gate_splits, gstride, gate_bias, w,
                                               w_dtype, w_next, w_next_dtype, x, N, H, eps, stream);
   else
     return IA_ERR_BAD_ARG;

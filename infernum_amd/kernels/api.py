@@ -1178,12 +1178,12 @@ def add_rows(h: torch.Tensor, table: torch.Tensor, index: torch.Tensor) -> torch
     return h
 
 
-def gated_norm_add(h: torch.Tensor, delta, gate: Optional[torch.Tensor], gate_bias: Optional[torch.Tensor],
+def gated_norm_add(h: torch.Tensor, delta, gate, gate_bias: Optional[torch.Tensor],
                    weight: torch.Tensor, eps: float, next_weight: Optional[torch.Tensor] = None,
                    x: Optional[torch.Tensor] = None) -> torch.Tensor:
     """d = delta * sigmoid(gate + gate_bias);  h += d * rsqrt(mean(d^2) + eps) * weight  (fp32, in place).  ``delta``: a
     tensor of h's shape in the activations' dtype or a :class:`SplitSum`; ``gate``: rows of at least H values (fp32 or
-    the activations' dtype) or None for no gate; ``x`` (optional, h's shape in the activations' dtype) receives
+    the activations' dtype), a :class:`SplitSum` of the logits, or None for no gate; ``x`` (optional, h's shape in the activations' dtype) receives
     rms_norm(h) * next_weight, or the new h itself without ``next_weight``."""
     split = isinstance(delta, SplitSum)
     d = delta.parts if split else delta
@@ -1196,9 +1196,15 @@ def gated_norm_add(h: torch.Tensor, delta, gate: Optional[torch.Tensor], gate_bi
         splits, d_rows = d.shape[0], d.shape[1]
     else:
         _need(d is not None and d.dtype in DTYPE_CODE and tuple(d.shape) == (N, H), "gated_norm_add: delta of h's shape")
-    if gate is not None:
+    g_splits, g_rows = 1, 0
+    if isinstance(gate, SplitSum):
+        gate = gate.parts
+        _need(gate.is_cuda and gate.shape[1] >= N and gate.shape[2] == H, "gated_norm_add: the gate's partial sums must be [S, >= N, H]")
+        g_splits, g_rows, g_stride = gate.shape[0], gate.shape[1], H
+    elif gate is not None:
         _rows(gate, H, "gated_norm_add gate")
         _need(gate.shape[0] >= N, "gated_norm_add: a gate row per row of h")
+        g_rows, g_stride = gate.shape[0], int(gate.stride(0))
     _f32(gate_bias, H, "gated_norm_add gate bias")
     for wt in (weight, next_weight):
         _need(wt is None or (wt.dtype in DTYPE_CODE and wt.numel() == H), f"gated_norm_add: weights of {H} values")
@@ -1208,7 +1214,7 @@ def gated_norm_add(h: torch.Tensor, delta, gate: Optional[torch.Tensor], gate_bi
               "gated_norm_add: x of h's shape in the activations' dtype")
     _ok(_core().ia_gated_norm_add(
         _p(h), _p(d), DTYPE_CODE[d.dtype], splits, d_rows, _p(gate), DTYPE_CODE[gate.dtype] if gate is not None else 0,
-        int(gate.stride(0)) if gate is not None else 0, _p(gate_bias), _p(weight), DTYPE_CODE[weight.dtype],
+        g_stride if gate is not None else 0, g_splits, g_rows, _p(gate_bias), _p(weight), DTYPE_CODE[weight.dtype],
         _p(next_weight), DTYPE_CODE[next_weight.dtype] if next_weight is not None else 0, _p(x), DTYPE_CODE[act], N, H,
         ctypes.c_float(eps), _stream()), "gated_norm_add")
     return h

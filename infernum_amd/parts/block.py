@@ -147,17 +147,22 @@ class SandwichBlock(Block):
         f32 = K.DTYPE_CODE[torch.float32]
         program.keep(post.weight, next_norm.weight if next_norm is not None else None,
                      gate.bias if gate is not None else None)
+        galts = logits.alts if logits is not None else [None]
         for alt in program.pending.alts:
             if not alt.splits and alt.dtype != self.rt.dtype:
                 raise K.KernelError("gated_norm_add: the delta must have the activations' dtype")
             code = f32 if alt.splits else program.act_code
-            program.op("core", "ia_gated_norm_add",
-                       [program.h, alt.where, code, alt.splits or 1, program.N, logits, f32, H,
-                        gate.bias if gate is not None else None, post.weight, K.DTYPE_CODE[post.weight.dtype],
-                        next_norm.weight if next_norm is not None else None,
-                        K.DTYPE_CODE[next_norm.weight.dtype] if next_norm is not None else 0,
-                        program.x if next_norm is not None else None, program.act_code, program.N, H, float(post.eps),
-                        STREAM], alt.when)
+            for galt in galts:                      # the gate's logits whole or as the parts of a split product
+                if galt is not None and galt.dtype != torch.float32:
+                    raise K.KernelError("gated_norm_add: the gate's logits must be fp32")
+                program.op("core", "ia_gated_norm_add",
+                           [program.h, alt.where, code, alt.splits or 1, program.N,
+                            galt.where if galt is not None else None, f32, H, (galt.splits or 1) if galt is not None else 1,
+                            program.N, gate.bias if gate is not None else None, post.weight,
+                            K.DTYPE_CODE[post.weight.dtype], next_norm.weight if next_norm is not None else None,
+                            K.DTYPE_CODE[next_norm.weight.dtype] if next_norm is not None else 0,
+                            program.x if next_norm is not None else None, program.act_code, program.N, H,
+                            float(post.eps), STREAM], alt.when & galt.when if galt is not None else alt.when)
         program.pending = None
 
     def native(self, program, view: CacheView) -> None:

@@ -36,15 +36,27 @@ class SigmoidLinearGate(Part):
     def load(self, tensors: Dict[str, torch.Tensor]) -> None:
         self.weight = tensors[self.name].contiguous()
         self.bias = tensors[self.bias_name].to(torch.float32).contiguous() if self.bias_name is not None else None
-        prepare_weights(self.rt, [(self.weight, None, False)])
+        prepare_weights(self.rt, [(self.weight, None, True), (self.weight, None, False)])
 
-    def logits(self, a: torch.Tensor) -> torch.Tensor:
-        """a [N, H] in the compute dtype -> G a, fp32 [N, H] (the bias is added where the sigmoid is taken)."""
-        return linear(a, self.weight, out_dtype=torch.float32, kernels=self.rt.kernels)
+    # up to so many rows the product's partial sums go on as they are (the kernel that takes the sigmoid adds them: a
+    # launch less a branch in steps of single tokens); above, the product leaves one matrix (a third of the bytes
+    # for that kernel to read where a long portion's product would be split)
+    SPLIT_UP_TO = 128
+
+    def logits(self, a: torch.Tensor):
+        """a [N, H] in the compute dtype -> G a, fp32 [N, H] or the partial sums of a split product (the kernel that
+        takes the sigmoid adds them, and the bias)."""
+        return linear(a, self.weight, out_dtype=torch.float32, keep_split=a.shape[0] <= self.SPLIT_UP_TO,
+                      kernels=self.rt.kernels)
 
     def emit_logits(self, program, key: str):
-        """The launches of :meth:`logits` on ``program.x``; returns the buffer [N, H] fp32."""
-        return emit_linear(program, program.x, program.N, self.weight, torch.float32, None, False, key, key).tensor()
+        """The launches of :meth:`logits` on ``program.x``; returns the Value [N, H] fp32, whole or in parts."""
+        from ..engine.program import Guard, Value
+        few = Guard.between(program.N, 0, self.SPLIT_UP_TO)
+        a = emit_linear(program, program.x, program.N, self.weight, torch.float32, None, True, key, key, when=few)
+        b = emit_linear(program, program.x, program.N, self.weight, torch.float32, None, False, key + ".whole",
+                        key + ".whole", when=~few)
+        return Value(self.hidden_size, list(a.alts) + list(b.alts))
 
 
 register_part("branch_gate", "sigmoid_linear", SigmoidLinearGate)

@@ -102,6 +102,12 @@ def test_gated_branch_norm(dtype, N, H, splits, gated, nxt):
     parts = torch.randn(max(splits, 1), N, H, generator=g)
     delta = parts.sum(0) if splits else _x(N, H, dtype, 4)
     gate, bias = torch.randn(N, H, generator=g) * 2, torch.randn(H, generator=g)
+    gate_parts = None
+    if gated and splits:                              # the gate's logits as the parts of a split product too
+        gate_parts = torch.randn(splits, N, H, generator=g)
+        gate = gate_parts[0].clone()
+        for k in range(1, splits):
+            gate = gate + gate_parts[k]
     w, w2 = torch.rand(H, generator=g) + 0.5, torch.rand(H, generator=g) + 0.5
     d = delta.double() * (PM.sigmoid(gate.double() + bias.double()) if gated else 1.0)
     want_h = h.double() + PM.rms_norm(d, w.double(), EPS)
@@ -109,7 +115,8 @@ def test_gated_branch_norm(dtype, N, H, splits, gated, nxt):
     hd = h.clone().to(DEV)
     xd = torch.empty((N, H), dtype=rt.dtype, device=DEV) if nxt else None
     dd = K.SplitSum(parts.to(DEV)) if splits else delta.to(DEV).to(rt.dtype)
-    K.gated_norm_add(hd, dd, gate.to(DEV) if gated else None, bias.to(DEV) if gated else None, w.to(DEV), EPS,
+    gd = K.SplitSum(gate_parts.to(DEV)) if gate_parts is not None else (gate.to(DEV) if gated else None)
+    K.gated_norm_add(hd, dd, gd, bias.to(DEV) if gated else None, w.to(DEV), EPS,
                      w2.to(DEV) if nxt else None, xd)
     assert rel_err(hd, want_h) <= 2e-5
     if nxt:
