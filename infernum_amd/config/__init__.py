@@ -3,5 +3,6 @@ from .llama import Llama3RopeScaling, LlamaConfig
 from .nesilorn import NesilornConfig
 from .rogizen import RogizenConfig
 from .malinex import MalinexConfig
+from .sikazen import SikazenConfig
 from .registry import (config_from_dict, load_config, model_spec_for, register_architecture, registered_architectures,
                        resolve_architecture)

@@ -8,7 +8,8 @@
 // Key pages are [num_pages, nkv, page_size, d], value pages [num_pages, nkv, d,
 // page_size]; block_tables[s, j / page_size] is the page of key j of sequence s.  The query of token n stands at positions[n] and
 // sees keys max(0, pos - window + 1) .. pos  (window 0: all keys from 0; window < 0: the keys of its own
-// chunk of -window positions, see ia_first_visible_key).
+// chunk of -window positions, see ia_first_visible_key).  sinks (nullable, fp32 [nh]): exp(sinks[h]) is added to
+// the softmax's denominator of head h; it has no key and no value.
 #include "common.h"
 
 #define AG_MAX_D 640
@@ -21,7 +22,7 @@ __global__ __launch_bounds__(64) void attn_generic_kernel(const T* __restrict__ 
                                                           const int* __restrict__ positions,
                                                           const int* __restrict__ block_tables, int bt_stride, int nh,
                                                           int nkv, int d, int page_size, int num_pages, float scale,
-                                                          int window) {
+                                                          int window, const float* __restrict__ sinks) {
   __shared__ float qs[AG_MAX_D];
   __shared__ float ps[64];
   __shared__ int rs[64];
@@ -83,6 +84,14 @@ __global__ __launch_bounds__(64) void attn_generic_kernel(const T* __restrict__ 
     __syncthreads();
     m = m_new;
   }
+  if (sinks) {          // a sink: exp(sink) more in the denominator, nothing in the sum
+    const float sk = sinks[h];
+    const float m_new = fmaxf(m, sk);
+    const float corr = expf(m - m_new);
+    l = l * corr + expf(sk - m_new);
+#pragma unroll
+    for (int c = 0; c < AG_MAX_D / 64; ++c) acc[c] *= corr;
+  }
   T* o = out + (size_t)n * out_row_stride + (size_t)h * d;
   const float inv_l = 1.0f / l;
 #pragma unroll
@@ -96,7 +105,7 @@ extern "C" int ia_attention_generic(const void* q, int q_row_stride, const void*
                                     void* out, int out_row_stride, int dtype, const int* token_seq,
                                     const int* positions, const int* block_tables, int bt_stride, int N, int nh,
                                     int nkv, int d, int page_size, int num_pages, float scale, int window,
-                                    hipStream_t stream) {
+                                    const float* sinks, hipStream_t stream) {
   if (N < 0 || nh <= 0 || nkv <= 0 || nh % nkv != 0 || d <= 0 || d > AG_MAX_D || page_size <= 0 || num_pages <= 0 ||
       bt_stride <= 0)
     return IA_ERR_BAD_ARG;
@@ -107,12 +116,12 @@ extern "C" int ia_attention_generic(const void* q, int q_row_stride, const void*
     attn_generic_kernel<float><<<grid, 64, 0, stream>>>((const float*)q, q_row_stride, (const float*)k_pages,
                                                         (const float*)v_pages, (float*)out, out_row_stride, token_seq,
                                                         positions, block_tables, bt_stride, nh, nkv, d, page_size,
-                                                        num_pages, scale, window);
+                                                        num_pages, scale, window, sinks);
   else if (dtype == IA_BF16)
     attn_generic_kernel<bf16_t><<<grid, 64, 0, stream>>>((const bf16_t*)q, q_row_stride, (const bf16_t*)k_pages,
                                                          (const bf16_t*)v_pages, (bf16_t*)out, out_row_stride,
                                                          token_seq, positions, block_tables, bt_stride, nh, nkv, d,
-                                                         page_size, num_pages, scale, window);
+                                                         page_size, num_pages, scale, window, sinks);
   else
     return IA_ERR_BAD_ARG;
   IA_LAUNCH_CHECK();

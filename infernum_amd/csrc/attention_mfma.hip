@@ -233,7 +233,7 @@ __global__ __launch_bounds__(WAVES * 64, ((WAVES == 4 && HD <= 128) ? 3 : 1)) vo
     const uint16_t* __restrict__ q, int q_row_stride, uint16_t* k_pages, uint16_t* v_pages,
     uint16_t* __restrict__ out, int out_row_stride, float* __restrict__ part_o, float* __restrict__ part_ml,
     const int* __restrict__ positions, const int* __restrict__ block_tables, int bt_stride, int nh, int nkv, int ps,
-    int num_pages, float scale_log2, int window, int num_splits, DecFused F) {
+    int num_pages, float scale_log2, int window, int num_splits, DecFused F, const float* __restrict__ sinks) {
   __shared__ float s_m[WAVES][16], s_l[WAVES][16];
   __shared__ f32x4 s_o[WAVES][NS][64];
   __shared__ int s_bt[DEC_BT_LDS];
@@ -427,7 +427,8 @@ __global__ __launch_bounds__(WAVES * 64, ((WAVES == 4 && HD <= 128) ? 3 : 1)) vo
 #pragma unroll
     for (int w = 1; w < WAVES; ++w) acc += s_o[w][n][lane];
     if (num_splits == 1) {
-      const float inv = 1.0f / L;
+      // a sink counts once, here or where the parts are joined
+      const float inv = 1.0f / (sinks ? L + exp2f(sinks[h] * 1.4426950408889634f - M) : L);
       uint2 wv;
       wv.x = (uint32_t)float_to_bf16_bits(acc[0] * inv) | ((uint32_t)float_to_bf16_bits(acc[1] * inv) << 16);
       wv.y = (uint32_t)float_to_bf16_bits(acc[2] * inv) | ((uint32_t)float_to_bf16_bits(acc[3] * inv) << 16);
@@ -449,7 +450,7 @@ __global__ __launch_bounds__(WAVES * 64, ((WAVES == 4 && HD <= 128) ? 3 : 1)) vo
 // the loads of the partial outputs do not wait for each other.
 extern "C" __global__ __launch_bounds__(64) void attn_decode_reduce_kernel(
     const float* __restrict__ part_o, const float* __restrict__ part_ml, uint16_t* __restrict__ out,
-    int out_row_stride, int nh, int num_splits) {
+    int out_row_stride, int nh, int num_splits, const float* __restrict__ sinks) {
   const int b = blockIdx.x / nh, h = blockIdx.x - b * nh, lane = threadIdx.x;
   const size_t rec0 = (size_t)blockIdx.x * num_splits;
   // the first parts' outputs are asked for together with the statistics, not after them
@@ -501,7 +502,7 @@ extern "C" __global__ __launch_bounds__(64) void attn_decode_reduce_kernel(
       }
     }
   }
-  const float inv = 1.0f / L;
+  const float inv = 1.0f / (sinks ? L + exp2f(sinks[h] * 1.4426950408889634f - M) : L);
 #pragma unroll
   for (int c = 0; c < (HD + 63) / 64; ++c) {
     const int dim = lane + 64 * c;
@@ -543,7 +544,7 @@ __global__ __launch_bounds__(4 * HGW * 64) void attn_prefill_kernel(
     const uint16_t* __restrict__ v_pages, uint16_t* __restrict__ out, int out_row_stride,
     const int* __restrict__ seq_starts, const int* __restrict__ seq_ctx, const int* __restrict__ block_tables,
     int bt_stride, const int* __restrict__ tiles, int nh, int nkv, int ps, int num_pages, float scale_log2,
-    int window, int paired) {
+    int window, int paired, const float* __restrict__ sinks) {
   __shared__ __attribute__((aligned(16))) uint16_t ks[2][PF_KT][PF_KROW];
   __shared__ __attribute__((aligned(16))) uint16_t vs[2][PF_SUBS][HD][PF_VROW];
   __shared__ int s_poison;
@@ -856,7 +857,9 @@ __global__ __launch_bounds__(4 * HGW * 64) void attn_prefill_kernel(
 #pragma unroll
   for (int c = 0; c < CT; ++c) {
     if (pos[c] < 0) continue;
-    const float inv = poison ? __uint_as_float(0x7fc00000u) : 1.0f / lacc[c][0];
+    float lsum = lacc[c][0];
+    if (sinks) lsum += exp2f(sinks[g * G + (hc * HGW + hgw) * CT + c] * 1.4426950408889634f - m[c]);
+    const float inv = poison ? __uint_as_float(0x7fc00000u) : 1.0f / lsum;
     uint16_t* orow = out + (size_t)(qstart + row) * out_row_stride +
                      (size_t)(g * G + (hc * HGW + hgw) * CT + c) * HD + 4 * qd;
 #pragma unroll
@@ -887,7 +890,7 @@ static int dec_check(int B, int nh, int nkv, int ps, int num_pages, int bt_strid
 extern "C" int ia_attn_decode(const void* q, int q_row_stride, const void* k_pages, const void* v_pages, void* out,
                               int out_row_stride, float* part_o, float* part_ml, const int* positions,
                               const int* block_tables, int bt_stride, int B, int nh, int nkv, int ps, int num_pages,
-                              float scale, int window, int num_splits, hipStream_t stream) {
+                              float scale, int window, int num_splits, const float* sinks, hipStream_t stream) {
   const int rc = dec_check(B, nh, nkv, ps, num_pages, bt_stride, num_splits, part_o, part_ml, out_row_stride);
   if (rc != IA_OK) return rc;
   if (q_row_stride & 7) return IA_ERR_UNSUPPORTED;
@@ -898,7 +901,7 @@ extern "C" int ia_attn_decode(const void* q, int q_row_stride, const void* k_pag
 #define DEC_LAUNCH(P2, W)                                                                                          \
   attn_decode_kernel<false, bf16_t, P2, W><<<grid, W * 64, 0, stream>>>(                                             \
       (const uint16_t*)q, q_row_stride, (uint16_t*)k_pages, (uint16_t*)v_pages, (uint16_t*)out, out_row_stride, part_o, \
-      part_ml, positions, block_tables, bt_stride, nh, nkv, ps, num_pages, scale_log2, window, num_splits, DecFused{})
+      part_ml, positions, block_tables, bt_stride, nh, nkv, ps, num_pages, scale_log2, window, num_splits, DecFused{}, sinks)
   const bool wide = dec_wide(B, nkv * HT, num_splits);
   if ((ps & (ps - 1)) == 0) {
     if (wide) DEC_LAUNCH(true, DEC_WAVES_FEW);
@@ -911,12 +914,14 @@ extern "C" int ia_attn_decode(const void* q, int q_row_stride, const void* k_pag
   IA_LAUNCH_CHECK();
   if (num_splits > 1) {
     attn_decode_reduce_kernel<<<B * nh, 64, 0, stream>>>(part_o, part_ml, (uint16_t*)out, out_row_stride, nh,
-                                                         num_splits);
+                                                         num_splits, sinks);
     IA_LAUNCH_CHECK();
   }
   return IA_OK;
 }
 
+// sinks (nullable, fp32 [nh], in all three launchers): exp(sinks[h]) is added to the softmax's denominator of
+// head h, once, where the sum over all keys is known.
 // The same with the rotation in front: row b of src is the QKV product of token b, [nh q heads | nkv k heads |
 // nkv v heads] (the k and v heads only with slots), in bf16 (src_dtype IA_BF16, src_splits 1) or as src_splits
 // partial sums in fp32, part s at src + s * src_rows * row_stride.  The first `rot` values of every q and k head
@@ -927,7 +932,7 @@ extern "C" int ia_attn_decode_fused(const void* src, int src_dtype, int src_spli
                                     void* v_pages, void* out, int out_row_stride, float* part_o, float* part_ml,
                                     const int* positions, const int* block_tables, int bt_stride, int B, int nh,
                                     int nkv, int ps, int num_pages, float scale, int window, int num_splits,
-                                    hipStream_t stream) {
+                                    const float* sinks, hipStream_t stream) {
   const int rc = dec_check(B, nh, nkv, ps, num_pages, bt_stride, num_splits, part_o, part_ml, out_row_stride);
   if (rc != IA_OK) return rc;
   if (!src || src_splits < 1 || src_rows < B || rot < 0 || rot > HD || (rot & 1)) return IA_ERR_BAD_ARG;
@@ -950,7 +955,7 @@ extern "C" int ia_attn_decode_fused(const void* src, int src_dtype, int src_spli
 #define DEC_FUSED_LAUNCH(TS, P2, W)                                                                                 \
   attn_decode_kernel<true, TS, P2, W><<<grid, W * 64, 0, stream>>>(                                                 \
       nullptr, 0, (uint16_t*)k_pages, (uint16_t*)v_pages, (uint16_t*)out, out_row_stride, part_o, part_ml, positions, \
-      block_tables, bt_stride, nh, nkv, ps, num_pages, scale_log2, window, num_splits, F)
+      block_tables, bt_stride, nh, nkv, ps, num_pages, scale_log2, window, num_splits, F, sinks)
 #define DEC_FUSED_WAVES(TS, P2)                       \
   do {                                                \
     if (wide) DEC_FUSED_LAUNCH(TS, P2, DEC_WAVES_FEW); \
@@ -969,7 +974,7 @@ extern "C" int ia_attn_decode_fused(const void* src, int src_dtype, int src_spli
   IA_LAUNCH_CHECK();
   if (num_splits > 1) {
     attn_decode_reduce_kernel<<<B * nh, 64, 0, stream>>>(part_o, part_ml, (uint16_t*)out, out_row_stride, nh,
-                                                         num_splits);
+                                                         num_splits, sinks);
     IA_LAUNCH_CHECK();
   }
   return IA_OK;
@@ -984,7 +989,7 @@ extern "C" int ia_attn_decode_fused(const void* src, int src_dtype, int src_spli
 extern "C" int ia_attn_prefill(const void* q, int q_row_stride, const void* k_pages, const void* v_pages, void* out,
                                int out_row_stride, const int* seq_starts, const int* seq_ctx, const int* block_tables,
                                int bt_stride, const int* tiles, int num_tiles, int nh, int nkv, int ps, int num_pages,
-                               float scale, int window, int launch_shape, hipStream_t stream) {
+                               float scale, int window, int launch_shape, const float* sinks, hipStream_t stream) {
   if (launch_shape < 0 || (launch_shape & ~(0xff | IA_PREFILL_PAIRED))) return IA_ERR_BAD_ARG;
   // under a window the rows of the two ends share no keys, and the keys between them may have no page any more:
   // rows are not paired then, whatever was asked for
@@ -1016,7 +1021,7 @@ extern "C" int ia_attn_prefill(const void* q, int q_row_stride, const void* k_pa
   attn_prefill_kernel<C, W, P2><<<grid, 4 * W * 64, 0, stream>>>(                                                 \
       (const uint16_t*)q, q_row_stride, (const uint16_t*)k_pages, (const uint16_t*)v_pages, (uint16_t*)out,       \
       out_row_stride, seq_starts, seq_ctx, block_tables, bt_stride, tiles, nh, nkv, ps, num_pages, scale_log2, window, \
-      paired)
+      paired, sinks)
 #define PF_LAUNCH(C, W)                      \
   do {                                       \
     if ((ps & (ps - 1)) == 0) PF_LAUNCH_P(C, W, true); \

@@ -48,6 +48,7 @@ CORE_SOURCES = [
     "seqmix.hip",
     "linear_attention.hip",
     "sigmoid_attention.hip",
+    "window_pool_attention.hip",
     "sampling.hip",
     "peaks.hip",
 ]

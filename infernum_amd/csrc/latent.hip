@@ -15,6 +15,7 @@
 // One workgroup a token.  src row: [H * (dn + dr) | rank | dr | ...]; dst row: (H + 2) heads of d = dr + rank.
 template <typename T>
 __global__ __launch_bounds__(256) void latent_prepare_kernel(const T* __restrict__ src, int src_stride,
+                                                             const T* __restrict__ lat_src, int lat_stride,
                                                              T* __restrict__ dst, int dst_stride,
                                                              const void* __restrict__ w, int w_dtype, int H, int dn,
                                                              int dr, int rank, float eps) {
@@ -26,7 +27,8 @@ __global__ __launch_bounds__(256) void latent_prepare_kernel(const T* __restrict
     const int h = i / dr, r = i - h * dr;
     o[(size_t)h * d + r] = s[(size_t)h * (dn + dr) + dn + r];
   }
-  const T* lat = s + (size_t)H * (dn + dr);
+  // the latent and the key's rotated part: behind the queries in their row, or rows of their own
+  const T* lat = lat_src ? lat_src + (size_t)n * lat_stride : s + (size_t)H * (dn + dr);
   float ss = 0.f;
   for (int i = threadIdx.x; i < rank; i += 256) {
     const float v = to_float(lat[i]);
@@ -47,17 +49,19 @@ __global__ __launch_bounds__(256) void latent_prepare_kernel(const T* __restrict
   }
 }
 
-extern "C" int ia_latent_prepare(const void* src, int src_stride, void* dst, int dst_stride, int dtype, const void* w,
-                                 int w_dtype, int N, int H, int dn, int dr, int rank, float eps, hipStream_t stream) {
-  if (N < 0 || H <= 0 || dn < 0 || dr < 0 || rank <= 0 || !(eps > 0.f) || src_stride < H * (dn + dr) + rank + dr ||
+extern "C" int ia_latent_prepare(const void* src, int src_stride, const void* lat, int lat_stride, void* dst,
+                                 int dst_stride, int dtype, const void* w, int w_dtype, int N, int H, int dn, int dr,
+                                 int rank, float eps, hipStream_t stream) {
+  if (N < 0 || H <= 0 || dn < 0 || dr < 0 || rank <= 0 || !(eps > 0.f) ||
+      src_stride < H * (dn + dr) + (lat ? 0 : rank + dr) || (lat && lat_stride < rank + dr) ||
       dst_stride < (H + 2) * (dr + rank))
     return IA_ERR_BAD_ARG;
   if (N == 0) return IA_OK;
   if (dtype == IA_F32)
-    latent_prepare_kernel<float><<<N, 256, 0, stream>>>((const float*)src, src_stride, (float*)dst, dst_stride, w,
+    latent_prepare_kernel<float><<<N, 256, 0, stream>>>((const float*)src, src_stride, (const float*)lat, lat_stride, (float*)dst, dst_stride, w,
                                                         w_dtype, H, dn, dr, rank, eps);
   else if (dtype == IA_BF16)
-    latent_prepare_kernel<bf16_t><<<N, 256, 0, stream>>>((const bf16_t*)src, src_stride, (bf16_t*)dst, dst_stride, w,
+    latent_prepare_kernel<bf16_t><<<N, 256, 0, stream>>>((const bf16_t*)src, src_stride, (const bf16_t*)lat, lat_stride, (bf16_t*)dst, dst_stride, w,
                                                          w_dtype, H, dn, dr, rank, eps);
   else
     return IA_ERR_BAD_ARG;

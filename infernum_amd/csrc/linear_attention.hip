@@ -49,7 +49,7 @@ __global__ __launch_bounds__(256) void gla_scan_kernel(
     int z_stride, const float* __restrict__ z_bias, float inv_tau, float q_scale, float* __restrict__ state,
     long state_stride, float* __restrict__ out, const int* __restrict__ seq_starts, const int* __restrict__ state_slots,
     int nh, int dim, int vdim, const int* __restrict__ tiles, int first_request, float* __restrict__ records,
-    long record_stride, float* __restrict__ decay) {
+    long record_stride, float* __restrict__ decay, int form) {
   extern __shared__ __attribute__((aligned(16))) float lds[];
   float* qs = lds;                                   // [TB][dim]
   float* ks = qs + GLA_TB * dim;                     // [TB][dim]
@@ -94,10 +94,12 @@ __global__ __launch_bounds__(256) void gla_scan_kernel(
       const size_t row = (size_t)(first + t0 + t);
       const T* pr = proj + row * proj_stride;
       qs[i] = to_float(pr[q_col + hd * dim + n]) * q_scale;
-      ks[i] = to_float(pr[k_col + hd * dim + n]);
       const float zz = z[row * z_stride + hd * dim + n];
-      // the tiles read decays that one kernel made of the logits before them; the walk over a request makes its own
-      as[i] = MODE != 0 ? zz : expf(gla_log_sigmoid(zz + (z_bias ? z_bias[hd * dim + n] : 0.f)) * inv_tau);
+      // the tiles read decays that one kernel made of the logits before them; the walk over a request makes its own.
+      // form 1: z holds the decays themselves, and what a channel does not keep it takes in: k = 1 - decay
+      const float a = (MODE != 0 || form == 1) ? zz : expf(gla_log_sigmoid(zz + (z_bias ? z_bias[hd * dim + n] : 0.f)) * inv_tau);
+      as[i] = a;
+      ks[i] = form == 1 ? 1.0f - a : to_float(pr[k_col + hd * dim + n]);
     }
     for (int i = tid; i < nt * GLA_PW; i += 256) {
       const int t = i / GLA_PW, c = slice * GLA_PW + (i - t * GLA_PW);
@@ -211,10 +213,10 @@ extern "C" long ia_gla_state_floats(int nh, int dim, int vdim) { return (long)nh
 
 // proj: rows of proj_stride values (code: their type) holding q (nh dim values from q_col), k (from k_col) and v (nh vdim
 // from v_col); z fp32 rows of z_stride values, z_bias (nullable) fp32 [nh dim]; out fp32 [N, nh vdim].
-extern "C" int ia_gla_scan(const void* proj, int code, int proj_stride, int q_col, int k_col, int v_col, const float* z,
+static int gla_scan_launch(const void* proj, int code, int proj_stride, int q_col, int k_col, int v_col, const float* z,
                            int z_stride, const float* z_bias, float tau, float q_scale, float* state, long state_stride,
                            float* out, const int* seq_starts, const int* state_slots, int B, int nh, int dim, int vdim,
-                           hipStream_t stream) {
+                           int form, hipStream_t stream) {
   if (B == 0) return IA_OK;
   if (!proj || !z || !state || !out || !seq_starts || !state_slots || B < 0 || nh <= 0 || dim <= 0 || vdim <= 0 ||
       !(tau > 0.f) || q_col < 0 || k_col < 0 || v_col < 0 || proj_stride < q_col + nh * dim ||
@@ -231,7 +233,7 @@ extern "C" int ia_gla_scan(const void* proj, int code, int proj_stride, int q_co
   gla_scan_kernel<T, KM, 0><<<grid, 256, lds, stream>>>((const T*)proj, proj_stride, q_col, k_col, v_col, z, z_stride, \
                                                         z_bias, 1.0f / tau, q_scale, state, state_stride, out,         \
                                                         seq_starts, state_slots, nh, dim, vdim, nullptr, 0, nullptr,   \
-                                                        0, nullptr)
+                                                        0, nullptr, form)
 #define IA_GLA_K(T)                       \
   do {                                    \
     if (per <= 4) IA_GLA(T, 4);           \
@@ -246,6 +248,23 @@ extern "C" int ia_gla_scan(const void* proj, int code, int proj_stride, int q_co
 #undef IA_GLA
   IA_LAUNCH_CHECK();
   return IA_OK;
+}
+
+extern "C" int ia_gla_scan(const void* proj, int code, int proj_stride, int q_col, int k_col, int v_col, const float* z,
+                           int z_stride, const float* z_bias, float tau, float q_scale, float* state, long state_stride,
+                           float* out, const int* seq_starts, const int* state_slots, int B, int nh, int dim, int vdim,
+                           hipStream_t stream) {
+  return gla_scan_launch(proj, code, proj_stride, q_col, k_col, v_col, z, z_stride, z_bias, tau, q_scale, state,
+                         state_stride, out, seq_starts, state_slots, B, nh, dim, vdim, 0, stream);
+}
+
+// The same recurrence with the decays given (f fp32 rows of f_stride values, each in [0, 1]) and k = 1 - f: a channel
+// takes in what it does not keep.  No factor on the queries.
+extern "C" int ia_hgrn2_scan(const void* proj, int code, int proj_stride, int q_col, int v_col, const float* f,
+                             int f_stride, float* state, long state_stride, float* out, const int* seq_starts,
+                             const int* state_slots, int B, int nh, int dim, int vdim, hipStream_t stream) {
+  return gla_scan_launch(proj, code, proj_stride, q_col, q_col, v_col, f, f_stride, nullptr, 1.0f, 1.0f, state,
+                         state_stride, out, seq_starts, state_slots, B, nh, dim, vdim, 1, stream);
 }
 
 // z <- alpha = exp(log_sigmoid(z + bias) / tau) in place, for the rows from request ``first_request``'s first on.
@@ -266,11 +285,11 @@ __global__ __launch_bounds__(256) void gla_decays_kernel(float* __restrict__ z, 
 // GLA_TILE among the request's rows) in any order, every tile of the requests first_request .. (and of no other)
 // once.  records: fp32 [num_tiles, record_stride >= ia_gla_state_floats]; decay: fp32 [num_tiles, nh, dim].  z has
 // num_rows rows; those of the requests first_request .. are left holding the decays, not the logits.
-extern "C" int ia_gla_chunked(const void* proj, int code, int proj_stride, int q_col, int k_col, int v_col, const float* z,
+static int gla_chunked_launch(const void* proj, int code, int proj_stride, int q_col, int k_col, int v_col, const float* z,
                               int z_stride, const float* z_bias, float tau, float q_scale, float* state,
                               long state_stride, float* out, const int* seq_starts, const int* state_slots,
                               const int* tiles, int num_tiles, int first_request, int num_rows, float* records, long record_stride, float* decay, int nh,
-                              int dim, int vdim, hipStream_t stream) {
+                              int dim, int vdim, int form, hipStream_t stream) {
   if (num_tiles == 0) return IA_OK;
   if (!proj || !z || !state || !out || !seq_starts || !state_slots || !tiles || !records || !decay || num_tiles < 0 || first_request < 0 || num_rows <= 0 ||
       nh <= 0 || dim <= 0 || vdim <= 0 || !(tau > 0.f) || q_col < 0 || k_col < 0 || v_col < 0 ||
@@ -287,7 +306,7 @@ extern "C" int ia_gla_chunked(const void* proj, int code, int proj_stride, int q
 #define IA_GLA(T, KM, MODE)                                                                                        \
   gla_scan_kernel<T, KM, MODE><<<grid, 256, lds, stream>>>(                                                        \
       (const T*)proj, proj_stride, q_col, k_col, v_col, z, z_stride, z_bias, 1.0f / tau, q_scale, state,           \
-      state_stride, out, seq_starts, state_slots, nh, dim, vdim, tiles, first_request, records, record_stride, decay)
+      state_stride, out, seq_starts, state_slots, nh, dim, vdim, tiles, first_request, records, record_stride, decay, form)
 #define IA_GLA_K(T, MODE)                       \
   do {                                          \
     if (per <= 4) IA_GLA(T, 4, MODE);           \
@@ -301,7 +320,7 @@ extern "C" int ia_gla_chunked(const void* proj, int code, int proj_stride, int q
     else IA_GLA_K(bf16_t, MODE);                   \
   } while (0)
   if (code != IA_F32 && code != IA_BF16) return IA_ERR_BAD_ARG;
-  {
+  if (form == 0) {
     const size_t most = (size_t)num_rows * nh * dim;
     gla_decays_kernel<<<(unsigned)((most + 255) / 256 < 262144 ? (most + 255) / 256 : 262144), 256, 0, stream>>>(
         const_cast<float*>(z), z_stride, z_bias, 1.0f / tau, seq_starts, first_request, num_rows, nh * dim);
@@ -316,6 +335,64 @@ extern "C" int ia_gla_chunked(const void* proj, int code, int proj_stride, int q
 #undef IA_GLA_T
 #undef IA_GLA_K
 #undef IA_GLA
+  IA_LAUNCH_CHECK();
+  return IA_OK;
+}
+
+extern "C" int ia_gla_chunked(const void* proj, int code, int proj_stride, int q_col, int k_col, int v_col, const float* z,
+                              int z_stride, const float* z_bias, float tau, float q_scale, float* state,
+                              long state_stride, float* out, const int* seq_starts, const int* state_slots,
+                              const int* tiles, int num_tiles, int first_request, int num_rows, float* records, long record_stride, float* decay, int nh,
+                              int dim, int vdim, hipStream_t stream) {
+  return gla_chunked_launch(proj, code, proj_stride, q_col, k_col, v_col, z, z_stride, z_bias, tau, q_scale, state,
+                            state_stride, out, seq_starts, state_slots, tiles, num_tiles, first_request, num_rows, records,
+                            record_stride, decay, nh, dim, vdim, 0, stream);
+}
+
+// ia_gla_chunked with the decays given and k = 1 - f (see ia_hgrn2_scan); f is left as it is.
+extern "C" int ia_hgrn2_chunked(const void* proj, int code, int proj_stride, int q_col, int v_col, const float* f,
+                                int f_stride, float* state, long state_stride, float* out, const int* seq_starts,
+                                const int* state_slots, const int* tiles, int num_tiles, int first_request, int num_rows,
+                                float* records, long record_stride, float* decay, int nh, int dim, int vdim,
+                                hipStream_t stream) {
+  return gla_chunked_launch(proj, code, proj_stride, q_col, q_col, v_col, f, f_stride, nullptr, 1.0f, 1.0f, state,
+                            state_stride, out, seq_starts, state_slots, tiles, num_tiles, first_request, num_rows, records,
+                            record_stride, decay, nh, dim, vdim, 1, stream);
+}
+
+// The gates of that recurrence, in place: the q columns of proj become silu(q) (in the activations' type), and
+// z (fp32 [N, cols], the logits of the forget gate) becomes f = lower + (1 - lower) sigmoid(z + bias).
+template <typename T>
+__global__ __launch_bounds__(256) void hgrn2_gates_kernel(T* __restrict__ proj, int proj_stride, int q_col,
+                                                          float* __restrict__ z, int z_stride,
+                                                          const float* __restrict__ bias, const float* __restrict__ lower,
+                                                          long total, int cols) {
+  const long i = (long)blockIdx.x * 256 + threadIdx.x;
+  if (i >= total) return;
+  const long n = i / cols;
+  const int c = (int)(i - n * cols);
+  T* q = proj + (size_t)n * proj_stride + q_col + c;
+  const float qv = to_float(*q);
+  *q = from_float<T>(qv / (1.0f + expf(-qv)));
+  float* zz = z + (size_t)n * z_stride + c;
+  const float lo = lower ? lower[c] : 0.f;
+  const float sg = 1.0f / (1.0f + expf(-(*zz + (bias ? bias[c] : 0.f))));
+  *zz = lo + (1.0f - lo) * sg;
+}
+
+extern "C" int ia_hgrn2_gates(void* proj, int code, int proj_stride, int q_col, float* z, int z_stride,
+                              const float* bias, const float* lower, int N, int cols, hipStream_t stream) {
+  if (N < 0 || cols <= 0 || q_col < 0 || proj_stride < q_col + cols || z_stride < cols) return IA_ERR_BAD_ARG;
+  if (N == 0) return IA_OK;
+  if (!proj || !z) return IA_ERR_BAD_ARG;
+  const long total = (long)N * cols;
+  const unsigned grid = (unsigned)((total + 255) / 256);
+  if (code == IA_F32)
+    hgrn2_gates_kernel<float><<<grid, 256, 0, stream>>>((float*)proj, proj_stride, q_col, z, z_stride, bias, lower, total, cols);
+  else if (code == IA_BF16)
+    hgrn2_gates_kernel<bf16_t><<<grid, 256, 0, stream>>>((bf16_t*)proj, proj_stride, q_col, z, z_stride, bias, lower, total, cols);
+  else
+    return IA_ERR_BAD_ARG;
   IA_LAUNCH_CHECK();
   return IA_OK;
 }
@@ -336,6 +413,10 @@ __global__ __launch_bounds__(256) void head_norm_gate_kernel(const float* __rest
   for (int i = lane; i < vdim; i += 64) ss = fmaf(orow[i], orow[i], ss);
   ss = wave_sum(ss);
   const float inv = 1.0f / sqrtf(ss / (float)vdim + eps);
+  if (!gate) {                       // no gate: the norm and the weight alone
+    for (int i = lane; i < vdim; i += 64) y[(size_t)pair * vdim + i] = from_float<T>(orow[i] * inv * w[i]);
+    return;
+  }
   const T* grow = gate + (size_t)n * gate_stride + gate_col + (size_t)hd * vdim;
   for (int i = lane; i < vdim; i += 64) {
     const float g = to_float(grow[i]);
@@ -345,10 +426,10 @@ __global__ __launch_bounds__(256) void head_norm_gate_kernel(const float* __rest
 
 extern "C" int ia_head_norm_gate(const float* o, const void* gate, int code, int gate_stride, int gate_col,
                                  const float* w, void* y, int N, int nh, int vdim, float eps, hipStream_t stream) {
-  if (N < 0 || nh <= 0 || vdim <= 0 || !(eps > 0.f) || gate_col < 0 || gate_stride < gate_col + nh * vdim)
+  if (N < 0 || nh <= 0 || vdim <= 0 || !(eps > 0.f) || (gate && (gate_col < 0 || gate_stride < gate_col + nh * vdim)))
     return IA_ERR_BAD_ARG;
   if (N == 0) return IA_OK;
-  if (!o || !gate || !w || !y) return IA_ERR_BAD_ARG;
+  if (!o || !w || !y) return IA_ERR_BAD_ARG;
   const long pairs = (long)N * nh;
   const long blocks = (pairs + 3) / 4;
   if (blocks > 0x7fffffffL) return IA_ERR_UNSUPPORTED;
@@ -367,4 +448,7 @@ extern "C" int ia_head_norm_gate(const float* o, const void* gate, int code, int
 #include "op_call.h"
 IA_OP(ia_gla_scan)
 IA_OP(ia_gla_chunked)
+IA_OP(ia_hgrn2_scan)
+IA_OP(ia_hgrn2_chunked)
+IA_OP(ia_hgrn2_gates)
 IA_OP(ia_head_norm_gate)

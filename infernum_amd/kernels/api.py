@@ -232,19 +232,27 @@ def activation(x: torch.Tensor, kind: str, out: Optional[torch.Tensor] = None) -
 
 
 def latent_prepare(proj: torch.Tensor, out: torch.Tensor, norm_weight: torch.Tensor, eps: float, H: int, dn: int,
-                   dr: int, rank: int) -> torch.Tensor:
+                   dr: int, rank: int, latent: Optional[torch.Tensor] = None, latent_col: int = 0) -> torch.Tensor:
     """From rows [H heads of (dn plain | dr rotated) query values | rank latent values | dr key values | ...]
     the rows [H heads of (dr | rank) | key (dr | rank) | value (dr | rank)] that the attention kernels take with
-    one key/value head: the rotated query parts at the heads' fronts (the rank places of the query heads are
+    one key/value head (``latent``: the rank latent values and dr key values stand in rows of their own, from column
+    ``latent_col`` on, and ``proj`` holds the queries alone): the rotated query parts at the heads' fronts (the rank places of the query heads are
     left for :func:`gemm_heads`), key = (k_rot, c), value = (0, c), c = RMSNorm(latent) * norm_weight."""
     _dev(proj, out, norm_weight)
     N = proj.shape[0]
     _need(proj.dim() == 2 and out.dim() == 2 and out.shape[0] == N and proj.dtype == out.dtype
           and proj.dtype in DTYPE_CODE, "latent_prepare: two matrices of one dtype with the same rows")
-    _need(proj.shape[1] >= H * (dn + dr) + rank + dr and out.shape[1] >= (H + 2) * (dr + rank),
-          "latent_prepare: rows too short for their heads")
+    _need(proj.shape[1] >= H * (dn + dr) + (0 if latent is not None else rank + dr)
+          and out.shape[1] >= (H + 2) * (dr + rank), "latent_prepare: rows too short for their heads")
+    lat_ptr, lat_stride = None, 0
+    if latent is not None:
+        _dev(latent)
+        _need(latent.dim() == 2 and latent.shape[0] == N and latent.dtype == proj.dtype and latent.stride(1) == 1
+              and latent_col >= 0 and latent.shape[1] >= latent_col + rank + dr, "latent_prepare: the latent's rows")
+        lat_ptr = ctypes.c_void_p(latent.data_ptr() + latent_col * latent.element_size())
+        lat_stride = int(latent.stride(0))
     _need(norm_weight.dtype in DTYPE_CODE and norm_weight.numel() == rank, f"latent_prepare: {rank} norm weights")
-    _ok(_core().ia_latent_prepare(_p(proj), proj.shape[1], _p(out), out.shape[1], DTYPE_CODE[out.dtype],
+    _ok(_core().ia_latent_prepare(_p(proj), proj.shape[1], lat_ptr, lat_stride, _p(out), out.shape[1], DTYPE_CODE[out.dtype],
                                   _p(norm_weight), DTYPE_CODE[norm_weight.dtype], N, H, dn, dr, rank,
                                   ctypes.c_float(eps), _stream()), "latent_prepare")
     return out
@@ -714,8 +722,9 @@ def _check_paged(qkv, k_pages, v_pages, out, block_tables, nh, nkv, d, what):
 
 def attention_generic(qkv: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, out: torch.Tensor,
                       token_seq: torch.Tensor, positions: torch.Tensor, block_tables: torch.Tensor, nh: int,
-                      nkv: int, d: int, scale: float, window: int = 0) -> None:
-    """Causal paged attention, one wave per (token, head), fp32 arithmetic.
+                      nkv: int, d: int, scale: float, window: int = 0, sinks: Optional[torch.Tensor] = None) -> None:
+    """Causal paged attention, one wave per (token, head), fp32 arithmetic.  ``sinks`` fp32 [nh]: exp(sinks[h]) is
+    added to the softmax's denominator of head h.
 
     qkv [N, >= nh*d]: the q heads of token n are the first nh*d values of row n.
     token_seq[n] is the row of block_tables of token n; positions[n] its position.
@@ -725,10 +734,11 @@ def attention_generic(qkv: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.T
     _i32(token_seq, N, "attention token_seq")
     _i32(positions, N, "attention positions")
     _need(0 < d <= GENERIC_MAX_HEAD_DIM, f"attention: head size must be at most {GENERIC_MAX_HEAD_DIM}")
+    _f32(sinks, nh, "attention sinks")
     _ok(_core().ia_attention_generic(_p(qkv), qkv.shape[1], _p(k_pages), _p(v_pages), _p(out), nh * d,
                                      DTYPE_CODE[out.dtype], _p(token_seq), _p(positions), _p(block_tables),
                                      block_tables.shape[1], N, nh, nkv, d, k_pages.shape[2], k_pages.shape[0],
-                                     ctypes.c_float(scale), int(window), _stream()), "attention_generic")
+                                     ctypes.c_float(scale), int(window), _p(sinks), _stream()), "attention_generic")
 
 
 def _attn(d: int) -> ctypes.CDLL:
@@ -778,7 +788,8 @@ def decode_splits(batch: int, nh: int, nkv: int, max_len: int, device: Optional[
 
 def attention_decode(qkv: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, out: torch.Tensor,
                      positions: torch.Tensor, block_tables: torch.Tensor, nh: int, nkv: int, d: int, scale: float,
-                     window: int, max_len: int, num_splits: Optional[int] = None) -> None:
+                     window: int, max_len: int, num_splits: Optional[int] = None,
+                     sinks: Optional[torch.Tensor] = None) -> None:
     """bf16 attention of B single tokens (row b of qkv: token b at positions[b]) over their pages, on MFMA.
 
     ``max_len`` bounds the positions (host side), and sets how many parts the keys are split into.
@@ -798,14 +809,15 @@ def attention_decode(qkv: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Te
         part_ml = torch.empty(B * nh * splits * 2, dtype=torch.float32, device=out.device)
     _ok(_attn(d).ia_attn_decode(_p(qkv), qkv.shape[1], _p(k_pages), _p(v_pages), _p(out), nh * d, _p(part_o),
                                 _p(part_ml), _p(positions), _p(block_tables), block_tables.shape[1], B, nh, nkv, ps,
-                                k_pages.shape[0], ctypes.c_float(scale), int(window), splits, _stream()),
+                                k_pages.shape[0], ctypes.c_float(scale), int(window), splits, _p(sinks), _stream()),
         "attention_decode")
 
 
 def attention_decode_rotating(qkv, positions: torch.Tensor, inv_freq: Optional[torch.Tensor], rot: int,
                               slots: Optional[torch.Tensor], k_pages: torch.Tensor, v_pages: torch.Tensor,
                               out: torch.Tensor, block_tables: torch.Tensor, nh: int, nkv: int, d: int, scale: float,
-                              window: int, max_len: int, num_splits: Optional[int] = None) -> None:
+                              window: int, max_len: int, num_splits: Optional[int] = None,
+                              sinks: Optional[torch.Tensor] = None) -> None:
     """:func:`rope_kv_append` and :func:`attention_decode` of B single tokens in one launch (the same bits).
 
     ``qkv`` is the QKV product of the tokens, [B, (nh + 2 nkv) d] in bf16 or a :class:`SplitSum` of it (with
@@ -850,8 +862,8 @@ def attention_decode_rotating(qkv, positions: torch.Tensor, inv_freq: Optional[t
         _p(src), DTYPE_CODE[src.dtype], src.shape[0] if split else 1, rows, row, _p(slots), _p(inv_freq),
         1 if (inv_freq is not None and inv_freq.dtype == torch.float64) else 0, rot if inv_freq is not None else 0,
         _p(k_pages), _p(v_pages), _p(out), nh * d, _p(part_o), _p(part_ml), _p(positions), _p(block_tables),
-        block_tables.shape[1], B, nh, nkv, ps, k_pages.shape[0], ctypes.c_float(scale), int(window), splits, _stream()),
-        "attention_decode_rotating")
+        block_tables.shape[1], B, nh, nkv, ps, k_pages.shape[0], ctypes.c_float(scale), int(window), splits, _p(sinks),
+        _stream()), "attention_decode_rotating")
 
 
 PREFILL_TILE_ROWS = 64      # query rows of a workgroup's tile in attention_prefill
@@ -861,7 +873,8 @@ PREFILL_PAIRED = 0x100      # in a launch shape: 32 rows from each end of a requ
 def attention_prefill(qkv: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, out: torch.Tensor,
                       seq_starts: torch.Tensor, seq_ctx: torch.Tensor, block_tables: torch.Tensor,
                       tiles: torch.Tensor, num_tiles: int, nh: int, nkv: int, d: int, scale: float,
-                      window: int, heads_per_workgroup: int = 0, paired: bool = False) -> None:
+                      window: int, heads_per_workgroup: int = 0, paired: bool = False,
+                      sinks: Optional[torch.Tensor] = None) -> None:
     """bf16 causal attention of portions of prompts over their pages, on MFMA.
 
     Request s brings rows seq_starts[s] .. seq_starts[s+1]-1 of qkv and had seq_ctx[s] tokens cached
@@ -883,7 +896,7 @@ def attention_prefill(qkv: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.T
     _ok(_attn(d).ia_attn_prefill(_p(qkv), qkv.shape[1], _p(k_pages), _p(v_pages), _p(out), nh * d, _p(seq_starts),
                                  _p(seq_ctx), _p(block_tables), block_tables.shape[1], _p(tiles), num_tiles, nh, nkv,
                                  ps, k_pages.shape[0], ctypes.c_float(scale), int(window),
-                                 int(heads_per_workgroup) | (PREFILL_PAIRED if paired else 0), _stream()),
+                                 int(heads_per_workgroup) | (PREFILL_PAIRED if paired else 0), _p(sinks), _stream()),
         "attention_prefill")
 
 
@@ -1342,19 +1355,206 @@ def gla_chunked(proj: torch.Tensor, q_col: int, k_col: int, v_col: int, z: torch
     return out
 
 
-def head_norm_gate(o: torch.Tensor, gate: torch.Tensor, gate_col: int, w: torch.Tensor, eps: float, nh: int, vdim: int,
-                   out: torch.Tensor) -> torch.Tensor:
+def head_norm_gate(o: torch.Tensor, gate: Optional[torch.Tensor], gate_col: int, w: torch.Tensor, eps: float, nh: int,
+                   vdim: int, out: torch.Tensor) -> torch.Tensor:
     """out = o / sqrt(mean(o^2) + eps) * w * silu(gate) with the mean over each head's vdim values: o fp32 [N, nh vdim],
     w fp32 [vdim] shared by the heads, gate rows holding nh vdim values from gate_col on."""
     N = o.shape[0]
     _need(o.is_cuda and o.dtype == torch.float32 and o.is_contiguous() and tuple(o.shape) == (N, nh * vdim),
           "head_norm_gate: o [N, nh vdim] fp32")
-    _rows(gate, gate_col + nh * vdim, "head_norm_gate gate")
     _f32(w, vdim, "head_norm_gate weight")
-    _need(out.is_cuda and out.is_contiguous() and tuple(out.shape) == (N, nh * vdim) and out.dtype == gate.dtype
-          and gate.shape[0] == N, "head_norm_gate: out [N, nh vdim] of the gate's dtype")
-    _ok(_core().ia_head_norm_gate(_p(o), _p(gate), DTYPE_CODE[gate.dtype], int(gate.stride(0)), gate_col, _p(w), _p(out),
-                                  N, nh, vdim, ctypes.c_float(eps), _stream()), "head_norm_gate")
+    _need(out.is_cuda and out.is_contiguous() and tuple(out.shape) == (N, nh * vdim) and out.dtype in DTYPE_CODE,
+          "head_norm_gate: out [N, nh vdim]")
+    if gate is not None:           # without a gate: the norm and the weight alone
+        _rows(gate, gate_col + nh * vdim, "head_norm_gate gate")
+        _need(out.dtype == gate.dtype and gate.shape[0] == N, "head_norm_gate: out of the gate's dtype")
+    _ok(_core().ia_head_norm_gate(_p(o), _p(gate), DTYPE_CODE[out.dtype], int(gate.stride(0)) if gate is not None else 0,
+                                  gate_col, _p(w), _p(out), N, nh, vdim, ctypes.c_float(eps), _stream()), "head_norm_gate")
+    return out
+
+
+# ------------------------------------------------------------ the recurrence with given decays (k = 1 - f)
+def hgrn2_gates(proj: torch.Tensor, q_col: int, z: torch.Tensor, bias: Optional[torch.Tensor],
+                lower: Optional[torch.Tensor]) -> None:
+    """In place: the ``z.shape[1]`` values of every row of ``proj`` from ``q_col`` on become silu of themselves, and
+    ``z`` (fp32 [N, C], logits) becomes lower + (1 - lower) sigmoid(z + bias)."""
+    N, C = z.shape
+    _rows(proj, q_col + C, "hgrn2_gates rows")
+    _need(z.is_cuda and z.dtype == torch.float32 and z.stride(1) == 1 and proj.shape[0] == N, "hgrn2_gates: z fp32 [N, C]")
+    _f32(bias, C, "hgrn2_gates bias")
+    _f32(lower, C, "hgrn2_gates lower")
+    _ok(_core().ia_hgrn2_gates(_p(proj), DTYPE_CODE[proj.dtype], int(proj.stride(0)), q_col, _p(z), int(z.stride(0)),
+                               _p(bias), _p(lower), N, C, _stream()), "hgrn2_gates")
+
+
+def hgrn2_scan(proj: torch.Tensor, q_col: int, v_col: int, f: torch.Tensor, state: torch.Tensor, out: torch.Tensor,
+               seq_starts: torch.Tensor, state_slots: torch.Tensor, nh: int, dim: int, vdim: int) -> torch.Tensor:
+    """:func:`gla_scan` with the decays given (``f`` fp32 [N, nh dim]) and k = 1 - f, no factor on the queries."""
+    N, B = proj.shape[0], state_slots.numel()
+    _rows(proj, max(q_col + nh * dim, v_col + nh * vdim), "hgrn2_scan rows")
+    _need(f.is_cuda and f.dtype == torch.float32 and f.dim() == 2 and f.stride(1) == 1 and f.shape[1] >= nh * dim
+          and f.shape[0] == N, "hgrn2_scan: f fp32 [N, nh dim]")
+    _need(out.is_cuda and out.dtype == torch.float32 and out.is_contiguous() and tuple(out.shape) == (N, nh * vdim),
+          "hgrn2_scan: out [N, nh vdim] fp32")
+    _i32(seq_starts, B + 1, "hgrn2_scan seq_starts")
+    _i32(state_slots, B, "hgrn2_scan state_slots")
+    stride = _state_rows(state, gla_state_floats(nh, dim, vdim), "hgrn2_scan")
+    _ok(_core().ia_hgrn2_scan(_p(proj), DTYPE_CODE[proj.dtype], int(proj.stride(0)), q_col, v_col, _p(f), int(f.stride(0)),
+                              _p(state), ctypes.c_long(stride), _p(out), _p(seq_starts), _p(state_slots), B, nh, dim, vdim,
+                              _stream()), "hgrn2_scan")
+    return out
+
+
+def hgrn2_chunked(proj: torch.Tensor, q_col: int, v_col: int, f: torch.Tensor, state: torch.Tensor, out: torch.Tensor,
+                  seq_starts: torch.Tensor, state_slots: torch.Tensor, tiles: torch.Tensor, num_tiles: int,
+                  first_request: int, nh: int, dim: int, vdim: int) -> torch.Tensor:
+    """:func:`gla_chunked` with the decays given and k = 1 - f."""
+    N = proj.shape[0]
+    _rows(proj, max(q_col + nh * dim, v_col + nh * vdim), "hgrn2_chunked rows")
+    _need(f.is_cuda and f.dtype == torch.float32 and f.dim() == 2 and f.stride(1) == 1 and f.shape[1] >= nh * dim
+          and f.shape[0] == N, "hgrn2_chunked: f fp32 [N, nh dim]")
+    _need(out.is_cuda and out.dtype == torch.float32 and out.is_contiguous() and tuple(out.shape) == (N, nh * vdim),
+          "hgrn2_chunked: out [N, nh vdim] fp32")
+    _dev(seq_starts, state_slots, tiles)
+    _need(seq_starts.dtype == torch.int32 and state_slots.dtype == torch.int32 and tiles.dtype == torch.int32
+          and tiles.is_contiguous() and tiles.numel() >= 2 * num_tiles, "hgrn2_chunked: int32 starts, slots and tiles")
+    floats = gla_state_floats(nh, dim, vdim)
+    stride = _state_rows(state, floats, "hgrn2_chunked")
+    records = torch.empty((max(num_tiles, 1), floats), dtype=torch.float32, device=out.device)
+    decay = torch.empty((max(num_tiles, 1), nh * dim), dtype=torch.float32, device=out.device)
+    _ok(_core().ia_hgrn2_chunked(_p(proj), DTYPE_CODE[proj.dtype], int(proj.stride(0)), q_col, v_col, _p(f),
+                                 int(f.stride(0)), _p(state), ctypes.c_long(stride), _p(out), _p(seq_starts),
+                                 _p(state_slots), _p(tiles), int(num_tiles), int(first_request), int(N), _p(records),
+                                 ctypes.c_long(floats), _p(decay), nh, dim, vdim, _stream()), "hgrn2_chunked")
+    return out
+
+
+# ------------------------------------------------ attention over a window of keys and pooled blocks before it
+WPA_MAX_HEAD_DIM = 640
+
+
+def wpa_pool_entries(page_size: int, pool: int) -> int:
+    """Pooled blocks a page of ``page_size`` positions can hold: those whose last position lies in the page."""
+    return (page_size - 1) // pool + 1
+
+
+def wpa_prepare(proj: torch.Tensor, bias: Optional[torch.Tensor], q_out: torch.Tensor, positions: torch.Tensor,
+                slots: torch.Tensor, freq: Optional[torch.Tensor], rot: int, unit_norm: bool, eps: float,
+                k_pages: torch.Tensor, v_pages: torch.Tensor, nh: int, nkv: int, d: int, dv: int) -> torch.Tensor:
+    """From rows [nh q heads of d | nkv k heads of d | nkv v heads of dv] (+ ``bias`` fp32): rotation of the first
+    ``rot`` values of every q and k head (value i with i + rot/2), then (``unit_norm``) every q and k head divided by
+    its root mean square; queries to ``q_out`` [N, nh d], keys to ``k_pages`` [pages, nkv, page, d] and values to
+    ``v_pages`` [pages, nkv, page, dv] at ``slots``."""
+    N = proj.shape[0]
+    row = (nh + nkv) * d + nkv * dv
+    _rows(proj, row, "wpa_prepare rows")
+    _rows(q_out, nh * d, "wpa_prepare q_out")
+    _need(q_out.dtype == proj.dtype and q_out.shape[0] == N and proj.dtype in DTYPE_CODE, "wpa_prepare: one dtype")
+    _f32(bias, row, "wpa_prepare bias")
+    _i32(positions, N, "wpa_prepare positions")
+    _i32(slots, N, "wpa_prepare slots")
+    if rot:
+        _need(freq is not None and freq.is_cuda and freq.dtype in (torch.float32, torch.float64)
+              and freq.numel() == rot // 2 and rot % 2 == 0 and rot <= d, "wpa_prepare: rot/2 frequencies, rot even, <= d")
+    num_pages, ps = k_pages.shape[0], k_pages.shape[2]
+    _need(k_pages.dtype == proj.dtype and v_pages.dtype == proj.dtype and k_pages.is_contiguous() and v_pages.is_contiguous()
+          and tuple(k_pages.shape) == (num_pages, nkv, ps, d) and tuple(v_pages.shape) == (num_pages, nkv, ps, dv),
+          "wpa_prepare: key pages [num_pages, nkv, page_size, d], value pages [num_pages, nkv, page_size, dv]")
+    _ok(_core().ia_wpa_prepare(_p(proj), int(proj.stride(0)), _p(bias), _p(q_out), int(q_out.stride(0)),
+                               DTYPE_CODE[proj.dtype], _p(positions), _p(slots), _p(freq if rot else None),
+                               1 if (rot and freq.dtype == torch.float64) else 0, int(rot), int(bool(unit_norm)),
+                               ctypes.c_float(eps), _p(k_pages), _p(v_pages), N, nh, nkv, d, dv, ps, num_pages, _stream()),
+        "wpa_prepare")
+    return q_out
+
+
+def wpa_pool(k_pages: torch.Tensor, v_pages: torch.Tensor, pk_pages: torch.Tensor, pv_pages: torch.Tensor,
+             token_seq: torch.Tensor, positions: torch.Tensor, bt_tokens: torch.Tensor, bt_pool: torch.Tensor,
+             pool: int) -> None:
+    """For every token of the step that is the last of a block of ``pool`` positions: the means of the block's keys
+    and values, read from the token pages, into the pooled pages ([pages, nkv, wpa_pool_entries, d | dv])."""
+    N = positions.numel()
+    num_pages, nkv, ps, d = k_pages.shape
+    dv = v_pages.shape[3]
+    E = wpa_pool_entries(ps, pool)
+    _need(tuple(pk_pages.shape[1:]) == (nkv, E, d) and tuple(pv_pages.shape[1:]) == (nkv, E, dv)
+          and pk_pages.dtype == k_pages.dtype == v_pages.dtype == pv_pages.dtype and pk_pages.is_contiguous()
+          and pv_pages.is_contiguous() and pk_pages.shape[0] == pv_pages.shape[0],
+          "wpa_pool: pooled pages [num_pages, nkv, entries, d | dv] of the token pages' dtype")
+    _i32(token_seq, N, "wpa_pool token_seq")
+    _need(bt_tokens.dtype == torch.int32 and bt_pool.dtype == torch.int32 and bt_tokens.dim() == 2 and bt_pool.dim() == 2
+          and bt_tokens.is_contiguous() and bt_pool.is_contiguous(), "wpa_pool: int32 block tables")
+    _dev(k_pages, v_pages, pk_pages, pv_pages, token_seq, positions, bt_tokens, bt_pool)
+    _ok(_core().ia_wpa_pool(_p(k_pages), _p(v_pages), _p(pk_pages), _p(pv_pages), DTYPE_CODE[k_pages.dtype], _p(token_seq),
+                            _p(positions), _p(bt_tokens), bt_tokens.shape[1], _p(bt_pool), bt_pool.shape[1], N, nkv, d, dv,
+                            ps, num_pages, pk_pages.shape[0], int(pool), _stream()), "wpa_pool")
+
+
+def wpa_attention(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, pk_pages: Optional[torch.Tensor],
+                  pv_pages: Optional[torch.Tensor], out: torch.Tensor, sinks: Optional[torch.Tensor],
+                  token_seq: torch.Tensor, positions: torch.Tensor, bt_tokens: torch.Tensor,
+                  bt_pool: Optional[torch.Tensor], nh: int, nkv: int, scale: float, window: int, pool: int) -> torch.Tensor:
+    """A query at position p sees keys p - window + 1 .. p (``window`` 0: all from 0) and, with ``pool`` > 0, every
+    block of ``pool`` positions that ends at or before p - window, through the means in the pooled pages; one softmax
+    over both, ``sinks`` fp32 [nh] in its denominator.  ``out`` [N, nh dv]."""
+    N = out.shape[0]
+    num_pages, _, ps, d = k_pages.shape
+    dv = v_pages.shape[3]
+    _rows(q, nh * d, "wpa_attention q")
+    _need(out.is_cuda and out.is_contiguous() and tuple(out.shape) == (N, nh * dv) and q.shape[0] == N
+          and q.dtype == out.dtype == k_pages.dtype == v_pages.dtype and q.dtype in DTYPE_CODE
+          and tuple(k_pages.shape) == (num_pages, nkv, ps, d) and tuple(v_pages.shape) == (num_pages, nkv, ps, dv)
+          and k_pages.is_contiguous() and v_pages.is_contiguous(), "wpa_attention: q, pages and out [N, nh dv] of one dtype")
+    _f32(sinks, nh, "wpa_attention sinks")
+    _i32(token_seq, N, "wpa_attention token_seq")
+    _i32(positions, N, "wpa_attention positions")
+    _need(bt_tokens.dtype == torch.int32 and bt_tokens.dim() == 2 and bt_tokens.is_contiguous(), "wpa_attention: block tables")
+    pooled = pool > 0 and window > 0
+    if pooled:
+        _need(pk_pages is not None and pv_pages is not None and bt_pool is not None and bt_pool.dtype == torch.int32
+              and bt_pool.is_contiguous() and pk_pages.dtype == q.dtype and pv_pages.dtype == q.dtype
+              and tuple(pk_pages.shape[1:]) == (nkv, wpa_pool_entries(ps, pool), d)
+              and tuple(pv_pages.shape[1:]) == (nkv, wpa_pool_entries(ps, pool), dv), "wpa_attention: pooled pages")
+    _dev(q, k_pages, v_pages, pk_pages, pv_pages, out, token_seq, positions, bt_tokens, bt_pool)
+    _ok(_core().ia_wpa_attention(_p(q), int(q.stride(0)), _p(k_pages), _p(v_pages), _p(pk_pages if pooled else None),
+                                 _p(pv_pages if pooled else None), _p(out), nh * dv, DTYPE_CODE[out.dtype], _p(sinks),
+                                 _p(token_seq), _p(positions), _p(bt_tokens), bt_tokens.shape[1],
+                                 _p(bt_pool if pooled else None), bt_pool.shape[1] if pooled else 0, N, nh, nkv, d, dv, ps,
+                                 num_pages, pk_pages.shape[0] if pooled else 0, ctypes.c_float(scale), int(window),
+                                 int(pool) if pooled else 0, _stream()), "wpa_attention")
+    return out
+
+
+def rms_rows(x: torch.Tensor, col: int, cols: int, weight: Optional[torch.Tensor], eps: float,
+             out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """out[n] = x[n, col : col + cols] / sqrt(mean of its squares + eps) * weight, in x's dtype."""
+    _rows(x, col + cols, "rms_rows x")
+    N = x.shape[0]
+    if out is None:
+        out = torch.empty((N, cols), dtype=x.dtype, device=x.device)
+    _need(out.is_cuda and out.dtype == x.dtype and tuple(out.shape) == (N, cols) and out.is_contiguous(), "rms_rows: out [N, cols]")
+    if weight is not None:
+        _need(weight.is_cuda and weight.dtype in DTYPE_CODE and weight.numel() == cols and weight.is_contiguous(),
+              "rms_rows: a weight a column")
+    _ok(_core().ia_rms_rows(ctypes.c_void_p(x.data_ptr() + col * x.element_size()), int(x.stride(0)), _p(weight),
+                            DTYPE_CODE[weight.dtype] if weight is not None else 0, _p(out), cols, DTYPE_CODE[x.dtype], N,
+                            cols, ctypes.c_float(eps), _stream()), "rms_rows")
+    return out
+
+
+def gelu_mul_rows(u: torch.Tensor, table: torch.Tensor, col: int, ids: torch.Tensor,
+                  out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """out[n, j] = gelu_tanh(u[n, j]) * table[ids[n], col + j]."""
+    N, C = u.shape
+    _need(u.is_cuda and u.is_contiguous() and u.dtype in DTYPE_CODE, "gelu_mul_rows: u [N, C]")
+    _need(table.is_cuda and table.dim() == 2 and table.is_contiguous() and table.dtype in DTYPE_CODE
+          and 0 <= col and col + C <= table.shape[1], "gelu_mul_rows: the table's rows are too short")
+    _i32(ids, N, "gelu_mul_rows ids")
+    if out is None:
+        out = torch.empty_like(u)
+    _need(out.is_cuda and out.is_contiguous() and out.dtype == u.dtype and out.shape == u.shape, "gelu_mul_rows: out like u")
+    _ok(_core().ia_gelu_mul_rows(_p(u), _p(out), DTYPE_CODE[u.dtype], _p(table), DTYPE_CODE[table.dtype], table.shape[1],
+                                 int(col), _p(ids), table.shape[0], N, C, _stream()), "gelu_mul_rows")
     return out
 
 

@@ -119,9 +119,10 @@ class DecoderModel:
         for (i, name, _), view in zip(self._cached(), views):
             per_entry[i][name] = view
         out = []
-        for named in per_entry:
+        for entry, named in zip(self.spec.schedule, per_entry):
             main = named.pop("mixer", None) or CacheView()
             main.others = named
+            main.pass_index = entry.pass_index
             out.append(main)
         return out
 

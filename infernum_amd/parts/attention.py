@@ -82,6 +82,9 @@ class Attention(Mixer):
                            and (self.qk_transform is None or getattr(self.qk_transform, "graph_safe", False)))
         self.w_qkv: Optional[torch.Tensor] = None
         self.w_o: Optional[torch.Tensor] = None
+        # fp32 [num_heads], or None: exp(sinks[h]) in the denominator of head h's softmax (a mixer that has sinks
+        # sets it when it loads; every attention kernel takes it)
+        self.sinks: Optional[torch.Tensor] = None
         self.rotate_in_attention = _decode_rotation == "attention"
         self.use_mfma = (kernels == "auto" and rt.dtype == torch.bfloat16 and rt.device.type == "cuda"
                          and K.attention_mfma_available(self.d))
@@ -161,7 +164,8 @@ class Attention(Mixer):
             out = torch.empty((n, nh * d), dtype=dtype, device=cache.k_pages.device)
             K.attention_decode_rotating(qkv, ctx.positions, self.position.inv_freq, self.position.rotary_dim,
                                         ctx.slots[g] if cache.writable else None, cache.k_pages, cache.v_pages, out,
-                                        ctx.block_tables[g], nh, nkv, d, self.scale, self.mask, self._span(ctx.max_total_len))
+                                        ctx.block_tables[g], nh, nkv, d, self.scale, self.mask, self._span(ctx.max_total_len),
+                                        sinks=self.sinks)
             return out
         q_out = None
         if isinstance(qkv, K.SplitSum):
@@ -217,7 +221,7 @@ class Attention(Mixer):
         T, N = program.T, program.N
         act, scale = program.act_code, float(self.scale)
         mfma = self.use_mfma and ps % 4 == 0
-        program.keep(k, v, inv_freq)
+        program.keep(k, v, inv_freq, self.sinks)
         bt, bt_cols = program.block_table(g), program.bt_cols(g)
         slots = program.slots(g) if writable else None
         out = program.buffer("attention.out", T * nh * d * program.act_bytes)
@@ -237,7 +241,8 @@ class Attention(Mixer):
             if mfma:
                 program.op(lib, "ia_attn_decode_fused",
                            [src, code, parts, N, row, slots, inv_freq, f64, rot, k, v, out, nh * d, part_o, part_ml,
-                            program.positions, bt, bt_cols, N, nh, nkv, ps, num_pages, scale, window, splits, STREAM],
+                            program.positions, bt, bt_cols, N, nh, nkv, ps, num_pages, scale, window, splits, self.sinks,
+                            STREAM],
                            alt.when & fused)
             q, q_stride = src, row
             if alt.splits:                   # partial sums: the rotated queries get a tensor of their own
@@ -283,14 +288,14 @@ class Attention(Mixer):
         k, v, g = view.k_pages, view.v_pages, view.group
         ps, num_pages = int(k.shape[2]), int(k.shape[0])
         T, act, scale = program.T, program.act_code, float(self.scale)
-        program.keep(k, v)
+        program.keep(k, v, self.sinks)
         bt, bt_cols = program.block_table(g), program.bt_cols(g)
         if out is None:
             out = program.buffer("attention.out", T * nh * d * program.act_bytes)
         if not (self.use_mfma and ps % 4 == 0):
             program.op("core", "ia_attention_generic",
                        [q, q_stride, k, v, out, nh * d, act, program.token_seq, program.positions, bt, bt_cols, program.N,
-                        nh, nkv, d, ps, num_pages, scale, window, STREAM], when)
+                        nh, nkv, d, ps, num_pages, scale, window, self.sinks, STREAM], when)
             return out
         lib = K._attn(d)
         records = T + 1024
@@ -300,10 +305,10 @@ class Attention(Mixer):
         tiles, num_tiles = program.row_tiles(K.PREFILL_TILE_ROWS)
         program.op(lib, "ia_attn_decode",
                    [q, q_stride, k, v, out, nh * d, part_o, part_ml, program.positions, bt, bt_cols, program.ND, nh,
-                    nkv, ps, num_pages, scale, window, splits, STREAM], when & Guard.between(program.ND, 1))
+                    nkv, ps, num_pages, scale, window, splits, self.sinks, STREAM], when & Guard.between(program.ND, 1))
         program.op(lib, "ia_attn_prefill",
                    [q, q_stride, k, v, out, nh * d, program.seq_starts, program.seq_ctx, bt, bt_cols, tiles, num_tiles,
-                    nh, nkv, ps, num_pages, scale, window, shape, STREAM], when & Guard.between(program.NP, 1))
+                    nh, nkv, ps, num_pages, scale, window, shape, self.sinks, STREAM], when & Guard.between(program.NP, 1))
         return out
 
     def _span(self, max_len: int) -> int:
@@ -316,12 +321,12 @@ class Attention(Mixer):
         bt = ctx.block_tables[cache.group]
         if not self.use_mfma or cache.k_pages.shape[2] % 4:
             K.attention_generic(qkv, cache.k_pages, cache.v_pages, out, ctx.token_seq, ctx.positions, bt, nh, nkv, d,
-                                self.scale, self.mask)
+                                self.scale, self.mask, sinks=self.sinks)
             return
         nd = ctx.num_decode
         if nd > 0:
             K.attention_decode(qkv[:nd], cache.k_pages, cache.v_pages, out[:nd], ctx.positions[:nd], bt[:nd], nh, nkv,
-                               d, self.scale, self.mask, self._span(ctx.max_total_len))
+                               d, self.scale, self.mask, self._span(ctx.max_total_len), sinks=self.sinks)
         if ctx.num_seqs > nd:
             key = ("prefill_launch_shape", nh, nkv, d, self.mask)
             hpw = ctx.extras.get(key)
@@ -330,7 +335,7 @@ class Attention(Mixer):
                                                                self.mask, qkv.device)
             tiles, num_tiles = ctx.row_tiles(K.PREFILL_TILE_ROWS)
             K.attention_prefill(qkv, cache.k_pages, cache.v_pages, out, ctx.seq_starts, ctx.seq_ctx, bt,
-                                tiles, num_tiles, nh, nkv, d, self.scale, self.mask, hpw)
+                                tiles, num_tiles, nh, nkv, d, self.scale, self.mask, hpw, sinks=self.sinks)
 
 
 register_part("mixer", "attention", Attention)

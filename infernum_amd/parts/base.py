@@ -49,17 +49,21 @@ class WeightSpec:
 class PageTensor:
     """One tensor of a page's payload.  ``shape`` is what one token stores; the page holds ``page_size`` tokens
     along a new axis put in at ``token_axis``: the pool is [num_pages, *shape[:token_axis], page_size,
-    *shape[token_axis:]].  ``dtype`` None: the compute type."""
+    *shape[token_axis:]].  ``dtype`` None: the compute type.  ``every`` e > 1: the page holds one entry for every e
+    positions, (page_size - 1) // e + 1 of them: the entry of the e positions that end at position t lies in t's
+    page at place (t % page_size) // e (a mixer that keeps something per block of positions)."""
 
     name: str
     shape: Tuple[int, ...]
     token_axis: int = 0
     dtype: Optional[torch.dtype] = None
+    every: int = 1
 
     def pool_shape(self, num_pages: int, page_size: int) -> Tuple[int, ...]:
         if not 0 <= self.token_axis <= len(self.shape):
             raise ValueError(f"page tensor {self.name!r}: token_axis {self.token_axis} is outside its shape {self.shape}")
-        return (num_pages,) + tuple(self.shape[:self.token_axis]) + (page_size,) + tuple(self.shape[self.token_axis:])
+        entries = page_size if self.every <= 1 else (page_size - 1) // self.every + 1
+        return (num_pages,) + tuple(self.shape[:self.token_axis]) + (entries,) + tuple(self.shape[self.token_axis:])
 
 
 @dataclass(frozen=True)
@@ -117,10 +121,13 @@ class LayerSpec:
 @dataclass(frozen=True)
 class ScheduleEntry:
     """One run of a layer.  ``cache_of`` names an earlier entry of the schedule
-    whose keys and values (or state) this run reads instead of writing its own."""
+    whose keys and values (or state) this run reads instead of writing its own.  ``pass_index``: which pass of a
+    stretch of layers that runs several times this run belongs to (0: the first, or no repetition); the run's
+    cache view carries it."""
 
     layer: int
     cache_of: Optional[int] = None
+    pass_index: int = 0
 
 
 @dataclass(frozen=True)
@@ -180,6 +187,7 @@ class CacheView:
     writable: bool = True
     state: Optional[torch.Tensor] = None
     others: Mapping[str, "CacheView"] = field(default_factory=dict)
+    pass_index: int = 0             # the schedule entry's: which pass of a repeated stretch of layers this run is
 
     @property
     def k_pages(self) -> Optional[torch.Tensor]:
@@ -422,8 +430,13 @@ class Block:
     def cached_parts(self) -> Dict[str, Part]:
         """The parts of this layer that keep something between steps (those with a ``cache_spec`` or a
         ``state_spec``), by name.  "mixer" gets the view that ``forward`` is handed; every other name is found in
-        that view's ``others``.  Each gets pages and state slots of its own from the cache manager."""
-        return {"mixer": self.mixer}
+        that view's ``others``.  Each gets pages and state slots of its own from the cache manager.  A mixer that
+        keeps a second kind of thing (in another group of pages than its keys) names it in ``cached_companions``."""
+        out = {"mixer": self.mixer}
+        companions = getattr(self.mixer, "cached_companions", None)
+        if companions is not None:
+            out.update(companions())
+        return out
 
     def native(self, program: Any, view: CacheView) -> None:
         """Write the arrangement into a step's program: its parts' operations in the order ``forward`` runs them

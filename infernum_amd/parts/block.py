@@ -19,6 +19,9 @@ feed_forward(f)).  The norms after the sublayers and the gates are extra parts (
 ``feed_forward_post_norm``: norms; ``mixer_gate``, ``feed_forward_gate``: category ``branch_gate``).  One kernel gates
 the branch, normalises it, adds it into the fp32 stream and, after the mixer, leaves the feed-forward's normalised
 input as well (``kernels.api.gated_norm_add``).
+
+``parallel``: h' = h + mixer(norm1(h)) + feed_forward(norm2(h)), both norms of the same stream; optionally a part
+that rewrites the stream at a later pass's entry and one that adds a token's own input after the sublayers.
 """
 from __future__ import annotations
 
@@ -180,6 +183,63 @@ class SandwichBlock(Block):
                               "sandwich.gate2")
 
 
+class ParallelBlock(Block):
+    """Mixer and feed-forward side by side, each behind a norm of its own of the SAME stream:
+    h' = h + mixer(norm1(h)) + feed_forward(norm2(h)); the feed-forward (with its norm) may be absent.  The two
+    results are added into the fp32 stream one after the other.  Extra parts: ``stream_in`` (category "stream_in")
+    rewrites the stream before the layer's norms, in every run of the layer but those of a repeated stretch's first
+    pass; ``token_input`` (category "token_input") adds to the finished stream after the sublayers."""
+    graph_safe = True
+
+    def forward(self, h: torch.Tensor, pending, ctx: StepContext, cache: CacheView):
+        from ..kernels import api as K
+        stream_in = self.extra.get("stream_in")
+        if stream_in is not None and cache.pass_index > 0:
+            stream_in.forward(h, pending, ctx)
+            pending = None
+        a = self.mixer.forward(self.mixer_norm.forward(h, pending), ctx, cache)
+        f = None
+        if self.feed_forward is not None:
+            f = self.feed_forward.forward(self.feed_forward_norm.forward(h, None), ctx)
+        K.stream_add(h, a)
+        if f is not None:
+            K.stream_add(h, f)
+        side = self.extra.get("token_input")
+        if side is not None:
+            side.forward(h, ctx)
+        return None
+
+    @staticmethod
+    def _emit_add(program, value) -> None:
+        from ..engine.program import STREAM
+        from ..kernels import api as K
+        f32 = K.DTYPE_CODE[torch.float32]
+        for alt in value.alts:
+            code = f32 if alt.splits else K.DTYPE_CODE[alt.dtype]
+            program.op("core", "ia_stream_add", [program.h, alt.where, code, alt.splits or 1, program.N,
+                                                 program.hidden_size, STREAM], alt.when)
+
+    def native(self, program, view: CacheView) -> None:
+        if type(self).forward is not ParallelBlock.forward:
+            return super().native(program, view)
+        if self.extra.get("stream_in") is not None and view.pass_index > 0:
+            self.extra["stream_in"].native(program, None)
+        self.mixer_norm.native(program, None)
+        self.mixer.native(program, view)
+        a, program.pending = program.pending, None
+        f = None
+        if self.feed_forward is not None:
+            self.feed_forward_norm.native(program, None)          # nothing pending: the norm of the same stream
+            self.feed_forward.native(program, None)
+            f, program.pending = program.pending, None
+        self._emit_add(program, a)
+        if f is not None:
+            self._emit_add(program, f)
+        if self.extra.get("token_input") is not None:
+            self.extra["token_input"].native(program, None)
+
+
 register_part("block", "prenorm", PreNormBlock)
+register_part("block", "parallel", ParallelBlock)
 register_part("block", "branchnorm", BranchNormBlock)
 register_part("block", "sandwich", SandwichBlock)

@@ -19,19 +19,26 @@ from .linear import emit_linear, linear
 
 
 EMBEDDING_OUTPUT = "embedding.out"
+EMBEDDING_OUTPUT_F32 = "embedding.out.f32"      # with keep_output="fp32": the rows as they entered the stream, unrounded
 
 
 class TokenEmbedding(Embedding):
     graph_safe = True
     def __init__(self, rt: Runtime, vocab_size: int, hidden_size: int, init_std: float = 0.02, scale: float = 1.0,
-                 name: str = "weight", keep_output: bool = False, position_table: Optional[Mapping[str, Any]] = None):
+                 name: str = "weight", keep_output: Any = False, position_table: Optional[Mapping[str, Any]] = None,
+                 extra_tables: Optional[Mapping[str, Any]] = None):
         """``position_table`` {name, rows, init_std}: a learned vector per position, added (unscaled) to the token's row;
         a position beyond its rows leaves NaN.  ``scale`` multiplies the looked-up row in fp32 (the table itself stays as stored: a head tied to it
         reads it unscaled); ``name`` is the table's local tensor name.  ``keep_output``: the rows as they leave
         here stay available to later parts of the step, rounded to the compute dtype (``EMBEDDING_OUTPUT`` in
-        ``ctx.extras``, or the program's buffer of that name)."""
+        ``ctx.extras``, or the program's buffer of that name); ``keep_output="fp32"`` keeps them unrounded
+        (``EMBEDDING_OUTPUT_F32``).  ``extra_tables`` {local name: {cols, init_std}}: further tables with a row per
+        token that this part owns and other parts read (they name the tensor as their fallback)."""
         super().__init__(rt)
-        self.keep_output = bool(keep_output)
+        self.keep_f32 = keep_output == "fp32"
+        self.keep_output = bool(keep_output) and not self.keep_f32
+        self.extra_tables = {k: dict(v) for k, v in (extra_tables or {}).items()}
+        self.tables: Dict[str, torch.Tensor] = {}
         self.vocab_size, self.hidden_size = int(vocab_size), int(hidden_size)
         self.init_std = init_std
         self.scale, self.name = float(scale), str(name)
@@ -44,12 +51,15 @@ class TokenEmbedding(Embedding):
         if self.position_table:
             out[self.position_table["name"]] = WeightSpec((int(self.position_table["rows"]), self.hidden_size),
                                                           ("normal", self.position_table.get("init_std", self.init_std)))
+        for name, t in self.extra_tables.items():
+            out[name] = WeightSpec((self.vocab_size, int(t["cols"])), ("normal", t.get("init_std", self.init_std)))
         return out
 
     def load(self, tensors: Dict[str, torch.Tensor]) -> None:
         self.table = tensors[self.name].contiguous()
         if self.position_table:
             self.pos_rows = tensors[self.position_table["name"]].contiguous()
+        self.tables = {name: tensors[name] for name in self.extra_tables}
 
     def forward(self, ctx: StepContext) -> torch.Tensor:
         h = torch.empty((ctx.num_tokens, self.hidden_size), dtype=torch.float32, device=self.table.device)
@@ -58,6 +68,8 @@ class TokenEmbedding(Embedding):
             K.add_rows(h, self.pos_rows, ctx.positions)
         if self.keep_output:
             ctx.extras[EMBEDDING_OUTPUT] = K.cast(h, self.rt.dtype)
+        if self.keep_f32:
+            ctx.extras[EMBEDDING_OUTPUT_F32] = K.cast(h, torch.float32, out=torch.empty_like(h))
         return h
 
     def native(self, program, view=None) -> None:
@@ -74,6 +86,10 @@ class TokenEmbedding(Embedding):
             kept = program.buffer(EMBEDDING_OUTPUT, program.T * self.hidden_size * program.act_bytes)
             program.op("core", "ia_cast", [program.h, K.DTYPE_CODE[torch.float32], kept, program.act_code,
                                            program.N * self.hidden_size, STREAM])
+        if self.keep_f32:
+            kept = program.buffer(EMBEDDING_OUTPUT_F32, program.T * self.hidden_size * 4)
+            f32 = K.DTYPE_CODE[torch.float32]
+            program.op("core", "ia_cast", [program.h, f32, kept, f32, program.N * self.hidden_size, STREAM])
         program.pending = None
 
 

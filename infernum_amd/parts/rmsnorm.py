@@ -10,6 +10,7 @@ Two options serve other arrangements with the same weight vector: ``unit_offset`
 :meth:`RMSNorm.add_normed`, the norm on a branch's output, h += norm(delta), which
 the ``branchnorm`` arrangement uses in place of ``forward``.  ``name`` is the
 tensor's local name ("weight" by default; "" when the prefix is the whole name).
+``scalar``: the stored weight is a single number for all values of a row.
 """
 from __future__ import annotations
 
@@ -24,8 +25,10 @@ from .base import Norm, Runtime, WeightSpec, register_part
 class RMSNorm(Norm):
     graph_safe = True
     def __init__(self, rt: Runtime, size: int, eps: float, init: tuple = ("ones",), unit_offset: bool = False,
-                 name: str = "weight"):
+                 name: str = "weight", scalar: bool = False):
+        """``scalar``: the file holds one number, which multiplies every value of the row."""
         super().__init__(rt)
+        self.scalar = bool(scalar)
         self.size = int(size)
         self.eps = float(eps)
         self.init = tuple(init)
@@ -35,10 +38,12 @@ class RMSNorm(Norm):
 
     def weights(self) -> Dict[str, WeightSpec]:
         # a norm weight stored in fp32 stays fp32; the kernel reads either
-        return {self.name: WeightSpec((self.size,), init=self.init, follows_compute_dtype=False)}
+        return {self.name: WeightSpec(() if self.scalar else (self.size,), init=self.init, follows_compute_dtype=False)}
 
     def load(self, tensors: Dict[str, torch.Tensor]) -> None:
         w = tensors[self.name].contiguous()
+        if self.scalar:             # the kernels read a weight a value: the one number, as often as the row is long
+            w = w.to(torch.float32).reshape(1).expand(self.size).contiguous()
         if self.unit_offset:
             w = (w.to(torch.float32) + 1.0).contiguous()       # 1 + w once, in fp32 (exact for a bf16 w)
         self.weight = w

@@ -19,6 +19,7 @@ original context, lo = max(floor(dim(fast)), 0), hi = min(ceil(dim(slow)), rot -
 r_i = clamp((i - lo) / max(hi - lo, 0.001), 0, 1), pair i turns at f_i / factor * r_i + f_i (1 - r_i); sine and cosine
 are both multiplied by ``magnitude`` = 0.1 ln(factor) + 1 (the reference's YaRN, infernum/src/rope.rs:91-120, has the
 same bands and correction).  ``pairing`` "neighbours" pairs value 2i with value 2i + 1 in place of i with i + rot/2.
+``linear`` scaling (key ``factor``) divides every frequency by the factor.
 
 Frequencies are formed and kept in float64; the rotation kernel forms the angle
 position * frequency in float64 too and brings it into [-pi, pi] before it takes
@@ -48,6 +49,9 @@ def rope_inverse_frequencies(rotary_dim: int, theta: float, scaling: Optional[Ma
             kind = scaling.get("rope_type")
             if kind == "yarn":
                 freqs.append(f)
+                continue
+            if kind == "linear":            # every frequency divided by the factor: positions counted in 1/factor steps
+                freqs.append(f / float(scaling["factor"]))
                 continue
             if kind != "llama3":
                 raise ValueError(f"rope scaling of type {kind!r} is not supported")

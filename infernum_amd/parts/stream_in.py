@@ -5,6 +5,8 @@ whose first width columns meet h.  A model that runs some of its layers several 
 which lets each pass see the tokens themselves again.  What a layer before left unadded (the pending delta) is added
 into h first; the product's operands are rounded to the compute dtype like any product's, its sums and the new stream
 are fp32.  The embedding must have been made with ``keep_output``.
+
+``add_embedding``: h <- h + e, nothing else.
 """
 from __future__ import annotations
 
@@ -14,7 +16,7 @@ import torch
 
 from ..kernels import api as K
 from .base import Part, Runtime, StepContext, WeightSpec, register_part
-from .embedding import EMBEDDING_OUTPUT
+from .embedding import EMBEDDING_OUTPUT, EMBEDDING_OUTPUT_F32
 from .linear import emit_linear, linear, prepare_weights
 
 
@@ -64,4 +66,35 @@ class ConcatLinearStreamIn(Part):
         emit_linear(program, both, N, self.weight, torch.float32, None, False, program.h, "stream_in")
 
 
+class AddEmbeddingStreamIn(Part):
+    """h <- h + e: the embedding's rows of the step's tokens, as they first entered the stream (fp32, unrounded),
+    are added again.  No tensors.  The embedding must have been made with ``keep_output="fp32"``."""
+    category = "stream_in"
+    graph_safe = True
+
+    def __init__(self, rt: Runtime, hidden_size: int):
+        super().__init__(rt)
+        self.hidden_size = int(hidden_size)
+
+    def forward(self, h: torch.Tensor, pending: Any, ctx: StepContext) -> None:
+        e = ctx.extras.get(EMBEDDING_OUTPUT_F32)
+        if e is None:
+            raise K.KernelError("add_embedding: the embedding did not keep its output (keep_output='fp32')")
+        if pending is not None:
+            K.stream_add(h, pending)
+        K.stream_add(h, e)
+
+    def native(self, program, view=None) -> None:
+        from ..engine.program import STREAM
+        H, N = self.hidden_size, program.N
+        f32 = K.DTYPE_CODE[torch.float32]
+        for alt in (program.pending.alts if program.pending is not None else []):
+            code = f32 if alt.splits else K.DTYPE_CODE[alt.dtype]
+            program.op("core", "ia_stream_add", [program.h, alt.where, code, alt.splits or 1, N, H, STREAM], alt.when)
+        program.pending = None
+        kept = program.buffer(EMBEDDING_OUTPUT_F32, program.T * H * 4)
+        program.op("core", "ia_stream_add", [program.h, kept, f32, 1, N, H, STREAM])
+
+
 register_part("stream_in", "concat_linear", ConcatLinearStreamIn)
+register_part("stream_in", "add_embedding", AddEmbeddingStreamIn)
