@@ -96,10 +96,12 @@ __global__ __launch_bounds__(256) void gla_scan_kernel(
       qs[i] = to_float(pr[q_col + hd * dim + n]) * q_scale;
       const float zz = z[row * z_stride + hd * dim + n];
       // the tiles read decays that one kernel made of the logits before them; the walk over a request makes its own.
-      // form 1: z holds the decays themselves, and what a channel does not keep it takes in: k = 1 - decay
+      // form 1: z holds the decays themselves, and z_bias is no bias but the rows of fp32 keys that go with them
+      // (what a channel takes in, 1 - decay, made where the decay was made and not as the difference of a number
+      // near one), laid out like z
       const float a = (MODE != 0 || form == 1) ? zz : expf(gla_log_sigmoid(zz + (z_bias ? z_bias[hd * dim + n] : 0.f)) * inv_tau);
       as[i] = a;
-      ks[i] = form == 1 ? 1.0f - a : to_float(pr[k_col + hd * dim + n]);
+      ks[i] = form == 1 ? z_bias[row * z_stride + hd * dim + n] : to_float(pr[k_col + hd * dim + n]);
     }
     for (int i = tid; i < nt * GLA_PW; i += 256) {
       const int t = i / GLA_PW, c = slice * GLA_PW + (i - t * GLA_PW);
@@ -258,12 +260,14 @@ extern "C" int ia_gla_scan(const void* proj, int code, int proj_stride, int q_co
                          state_stride, out, seq_starts, state_slots, B, nh, dim, vdim, 0, stream);
 }
 
-// The same recurrence with the decays given (f fp32 rows of f_stride values, each in [0, 1]) and k = 1 - f: a channel
-// takes in what it does not keep.  No factor on the queries.
+// The same recurrence with the decays given (f fp32 rows of f_stride values, each in [0, 1]) and the keys with them
+// (k fp32, laid out like f: 1 - f, what a channel takes in because it does not keep it).  No factor on the queries.
 extern "C" int ia_hgrn2_scan(const void* proj, int code, int proj_stride, int q_col, int v_col, const float* f,
-                             int f_stride, float* state, long state_stride, float* out, const int* seq_starts,
-                             const int* state_slots, int B, int nh, int dim, int vdim, hipStream_t stream) {
-  return gla_scan_launch(proj, code, proj_stride, q_col, q_col, v_col, f, f_stride, nullptr, 1.0f, 1.0f, state,
+                             const float* k, int f_stride, float* state, long state_stride, float* out,
+                             const int* seq_starts, const int* state_slots, int B, int nh, int dim, int vdim,
+                             hipStream_t stream) {
+  if (!k) return IA_ERR_BAD_ARG;
+  return gla_scan_launch(proj, code, proj_stride, q_col, q_col, v_col, f, f_stride, k, 1.0f, 1.0f, state,
                          state_stride, out, seq_starts, state_slots, B, nh, dim, vdim, 1, stream);
 }
 
@@ -349,22 +353,24 @@ extern "C" int ia_gla_chunked(const void* proj, int code, int proj_stride, int q
                             record_stride, decay, nh, dim, vdim, 0, stream);
 }
 
-// ia_gla_chunked with the decays given and k = 1 - f (see ia_hgrn2_scan); f is left as it is.
+// ia_gla_chunked with the decays and the keys given (see ia_hgrn2_scan); f is left as it is.
 extern "C" int ia_hgrn2_chunked(const void* proj, int code, int proj_stride, int q_col, int v_col, const float* f,
-                                int f_stride, float* state, long state_stride, float* out, const int* seq_starts,
+                                const float* k, int f_stride, float* state, long state_stride, float* out, const int* seq_starts,
                                 const int* state_slots, const int* tiles, int num_tiles, int first_request, int num_rows,
                                 float* records, long record_stride, float* decay, int nh, int dim, int vdim,
                                 hipStream_t stream) {
-  return gla_chunked_launch(proj, code, proj_stride, q_col, q_col, v_col, f, f_stride, nullptr, 1.0f, 1.0f, state,
+  if (!k) return IA_ERR_BAD_ARG;
+  return gla_chunked_launch(proj, code, proj_stride, q_col, q_col, v_col, f, f_stride, k, 1.0f, 1.0f, state,
                             state_stride, out, seq_starts, state_slots, tiles, num_tiles, first_request, num_rows, records,
                             record_stride, decay, nh, dim, vdim, 1, stream);
 }
 
-// The gates of that recurrence, in place: the q columns of proj become silu(q) (in the activations' type), and
-// z (fp32 [N, cols], the logits of the forget gate) becomes f = lower + (1 - lower) sigmoid(z + bias).
+// The gates of that recurrence: the q columns of proj become silu(q) in place (in the activations' type), z (fp32
+// [N, cols], the logits of the forget gate) becomes f = lower + (1 - lower) sigmoid(z + bias) in place, and k (laid
+// out like z) gets 1 - f = (1 - lower) sigmoid(-(z + bias)), which is exact where f is within rounding of one.
 template <typename T>
 __global__ __launch_bounds__(256) void hgrn2_gates_kernel(T* __restrict__ proj, int proj_stride, int q_col,
-                                                          float* __restrict__ z, int z_stride,
+                                                          float* __restrict__ z, float* __restrict__ k, int z_stride,
                                                           const float* __restrict__ bias, const float* __restrict__ lower,
                                                           long total, int cols) {
   const long i = (long)blockIdx.x * 256 + threadIdx.x;
@@ -376,21 +382,22 @@ __global__ __launch_bounds__(256) void hgrn2_gates_kernel(T* __restrict__ proj, 
   *q = from_float<T>(qv / (1.0f + expf(-qv)));
   float* zz = z + (size_t)n * z_stride + c;
   const float lo = lower ? lower[c] : 0.f;
-  const float sg = 1.0f / (1.0f + expf(-(*zz + (bias ? bias[c] : 0.f))));
-  *zz = lo + (1.0f - lo) * sg;
+  const float x = *zz + (bias ? bias[c] : 0.f);
+  *zz = lo + (1.0f - lo) * (1.0f / (1.0f + expf(-x)));
+  k[(size_t)n * z_stride + c] = (1.0f - lo) * (1.0f / (1.0f + expf(x)));
 }
 
-extern "C" int ia_hgrn2_gates(void* proj, int code, int proj_stride, int q_col, float* z, int z_stride,
+extern "C" int ia_hgrn2_gates(void* proj, int code, int proj_stride, int q_col, float* z, float* k, int z_stride,
                               const float* bias, const float* lower, int N, int cols, hipStream_t stream) {
   if (N < 0 || cols <= 0 || q_col < 0 || proj_stride < q_col + cols || z_stride < cols) return IA_ERR_BAD_ARG;
   if (N == 0) return IA_OK;
-  if (!proj || !z) return IA_ERR_BAD_ARG;
+  if (!proj || !z || !k) return IA_ERR_BAD_ARG;
   const long total = (long)N * cols;
   const unsigned grid = (unsigned)((total + 255) / 256);
   if (code == IA_F32)
-    hgrn2_gates_kernel<float><<<grid, 256, 0, stream>>>((float*)proj, proj_stride, q_col, z, z_stride, bias, lower, total, cols);
+    hgrn2_gates_kernel<float><<<grid, 256, 0, stream>>>((float*)proj, proj_stride, q_col, z, k, z_stride, bias, lower, total, cols);
   else if (code == IA_BF16)
-    hgrn2_gates_kernel<bf16_t><<<grid, 256, 0, stream>>>((bf16_t*)proj, proj_stride, q_col, z, z_stride, bias, lower, total, cols);
+    hgrn2_gates_kernel<bf16_t><<<grid, 256, 0, stream>>>((bf16_t*)proj, proj_stride, q_col, z, k, z_stride, bias, lower, total, cols);
   else
     return IA_ERR_BAD_ARG;
   IA_LAUNCH_CHECK();

@@ -1375,21 +1375,29 @@ def head_norm_gate(o: torch.Tensor, gate: Optional[torch.Tensor], gate_col: int,
 
 # ------------------------------------------------------------ the recurrence with given decays (k = 1 - f)
 def hgrn2_gates(proj: torch.Tensor, q_col: int, z: torch.Tensor, bias: Optional[torch.Tensor],
-                lower: Optional[torch.Tensor]) -> None:
+                lower: Optional[torch.Tensor], k: Optional[torch.Tensor] = None) -> torch.Tensor:
     """In place: the ``z.shape[1]`` values of every row of ``proj`` from ``q_col`` on become silu of themselves, and
-    ``z`` (fp32 [N, C], logits) becomes lower + (1 - lower) sigmoid(z + bias)."""
+    ``z`` (fp32 [N, C], logits) becomes f = lower + (1 - lower) sigmoid(z + bias).  Returns ``k`` (fp32, like z):
+    1 - f, made as (1 - lower) sigmoid(-(z + bias))."""
     N, C = z.shape
+    if k is None:
+        k = torch.empty_like(z)
+    _need(k.is_cuda and k.dtype == torch.float32 and k.shape == z.shape and k.stride() == z.stride(), "hgrn2_gates: k like z")
     _rows(proj, q_col + C, "hgrn2_gates rows")
     _need(z.is_cuda and z.dtype == torch.float32 and z.stride(1) == 1 and proj.shape[0] == N, "hgrn2_gates: z fp32 [N, C]")
     _f32(bias, C, "hgrn2_gates bias")
     _f32(lower, C, "hgrn2_gates lower")
-    _ok(_core().ia_hgrn2_gates(_p(proj), DTYPE_CODE[proj.dtype], int(proj.stride(0)), q_col, _p(z), int(z.stride(0)),
+    _ok(_core().ia_hgrn2_gates(_p(proj), DTYPE_CODE[proj.dtype], int(proj.stride(0)), q_col, _p(z), _p(k), int(z.stride(0)),
                                _p(bias), _p(lower), N, C, _stream()), "hgrn2_gates")
+    return k
 
 
-def hgrn2_scan(proj: torch.Tensor, q_col: int, v_col: int, f: torch.Tensor, state: torch.Tensor, out: torch.Tensor,
-               seq_starts: torch.Tensor, state_slots: torch.Tensor, nh: int, dim: int, vdim: int) -> torch.Tensor:
-    """:func:`gla_scan` with the decays given (``f`` fp32 [N, nh dim]) and k = 1 - f, no factor on the queries."""
+def hgrn2_scan(proj: torch.Tensor, q_col: int, v_col: int, f: torch.Tensor, k: torch.Tensor, state: torch.Tensor,
+               out: torch.Tensor, seq_starts: torch.Tensor, state_slots: torch.Tensor, nh: int, dim: int,
+               vdim: int) -> torch.Tensor:
+    """:func:`gla_scan` with the decays (``f`` fp32 [N, nh dim]) and the keys (``k`` = 1 - f, like f) given, no factor
+    on the queries."""
+    _need(k.is_cuda and k.dtype == torch.float32 and k.shape == f.shape and k.stride() == f.stride(), "hgrn2_scan: k like f")
     N, B = proj.shape[0], state_slots.numel()
     _rows(proj, max(q_col + nh * dim, v_col + nh * vdim), "hgrn2_scan rows")
     _need(f.is_cuda and f.dtype == torch.float32 and f.dim() == 2 and f.stride(1) == 1 and f.shape[1] >= nh * dim
@@ -1399,16 +1407,17 @@ def hgrn2_scan(proj: torch.Tensor, q_col: int, v_col: int, f: torch.Tensor, stat
     _i32(seq_starts, B + 1, "hgrn2_scan seq_starts")
     _i32(state_slots, B, "hgrn2_scan state_slots")
     stride = _state_rows(state, gla_state_floats(nh, dim, vdim), "hgrn2_scan")
-    _ok(_core().ia_hgrn2_scan(_p(proj), DTYPE_CODE[proj.dtype], int(proj.stride(0)), q_col, v_col, _p(f), int(f.stride(0)),
+    _ok(_core().ia_hgrn2_scan(_p(proj), DTYPE_CODE[proj.dtype], int(proj.stride(0)), q_col, v_col, _p(f), _p(k), int(f.stride(0)),
                               _p(state), ctypes.c_long(stride), _p(out), _p(seq_starts), _p(state_slots), B, nh, dim, vdim,
                               _stream()), "hgrn2_scan")
     return out
 
 
-def hgrn2_chunked(proj: torch.Tensor, q_col: int, v_col: int, f: torch.Tensor, state: torch.Tensor, out: torch.Tensor,
-                  seq_starts: torch.Tensor, state_slots: torch.Tensor, tiles: torch.Tensor, num_tiles: int,
-                  first_request: int, nh: int, dim: int, vdim: int) -> torch.Tensor:
-    """:func:`gla_chunked` with the decays given and k = 1 - f."""
+def hgrn2_chunked(proj: torch.Tensor, q_col: int, v_col: int, f: torch.Tensor, k: torch.Tensor, state: torch.Tensor,
+                  out: torch.Tensor, seq_starts: torch.Tensor, state_slots: torch.Tensor, tiles: torch.Tensor,
+                  num_tiles: int, first_request: int, nh: int, dim: int, vdim: int) -> torch.Tensor:
+    """:func:`gla_chunked` with the decays and the keys given (see :func:`hgrn2_scan`)."""
+    _need(k.is_cuda and k.dtype == torch.float32 and k.shape == f.shape and k.stride() == f.stride(), "hgrn2_chunked: k like f")
     N = proj.shape[0]
     _rows(proj, max(q_col + nh * dim, v_col + nh * vdim), "hgrn2_chunked rows")
     _need(f.is_cuda and f.dtype == torch.float32 and f.dim() == 2 and f.stride(1) == 1 and f.shape[1] >= nh * dim
@@ -1422,7 +1431,7 @@ def hgrn2_chunked(proj: torch.Tensor, q_col: int, v_col: int, f: torch.Tensor, s
     stride = _state_rows(state, floats, "hgrn2_chunked")
     records = torch.empty((max(num_tiles, 1), floats), dtype=torch.float32, device=out.device)
     decay = torch.empty((max(num_tiles, 1), nh * dim), dtype=torch.float32, device=out.device)
-    _ok(_core().ia_hgrn2_chunked(_p(proj), DTYPE_CODE[proj.dtype], int(proj.stride(0)), q_col, v_col, _p(f),
+    _ok(_core().ia_hgrn2_chunked(_p(proj), DTYPE_CODE[proj.dtype], int(proj.stride(0)), q_col, v_col, _p(f), _p(k),
                                  int(f.stride(0)), _p(state), ctypes.c_long(stride), _p(out), _p(seq_starts),
                                  _p(state_slots), _p(tiles), int(num_tiles), int(first_request), int(N), _p(records),
                                  ctypes.c_long(floats), _p(decay), nh, dim, vdim, _stream()), "hgrn2_chunked")

@@ -73,6 +73,8 @@ def sikazen_model_spec(cfg: SikazenConfig, init_std: float = 0.05) -> ModelSpec:
         layers=layers, schedule=[ScheduleEntry(i, pass_index=t) for i, t in runs],
         final_norm=norm("final.norm"),
         head=PartSpec("linear", {"vocab_size": cfg.vocab, "hidden_size": W, "name": "", "init_std": W ** -0.5}, "head"),
+        # a layer without a feed-forward has no use for a second norm, whether the file holds one or not
+        ignored_tensors=tuple(f"l{i}.norm2" for i, layer in enumerate(cfg.layers) if layer.mlp is None),
     )
 
 

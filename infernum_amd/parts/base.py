@@ -144,6 +144,8 @@ class ModelSpec:
     max_position: int = 0
     bos_token_id: Optional[int] = None
     eos_token_id: Optional[int] = None
+    # names (patterns of fnmatch) of tensors that a file may hold and no part reads
+    ignored_tensors: Sequence[str] = ()
 
 
 # -------------------------------------------------------------------- run time

@@ -11,7 +11,8 @@ multiplied by a weight that the heads share; the heads, concatenated, are projec
 It is the recurrence of gated linear attention with the decays given and the keys 1 - f, and runs on that mixer's
 kernels (token after token for single tokens, tiles of rows side by side for portions of prompts) in their form for
 given decays; a request keeps every head's S in one state slot of fp32 values.  The gate's logits leave their
-product in fp32; the sigmoid, the bound, 1 - f, the state and the norm are fp32 whatever the activations' type.
+product in fp32; the sigmoid, the bound, 1 - f, the state and the norm are fp32 whatever the activations' type, and
+1 - f is made as (1 - l) sigmoid(-(Wf x + b)), not as the difference of an f that rounding has moved to one.
 """
 from __future__ import annotations
 
@@ -73,15 +74,15 @@ class Hgrn2(Mixer):
         state = self._state(cache)
         proj = linear(x, self.w_in, kernels=self.rt.kernels)                            # [n, q | v]
         f = linear(x, self.w_f, out_dtype=torch.float32, kernels=self.rt.kernels)       # the gate's logits, then the gate
-        K.hgrn2_gates(proj, self.q_col, f, self.b_f, self.lower)
+        k = K.hgrn2_gates(proj, self.q_col, f, self.b_f, self.lower)
         o = torch.empty((n, self.nv), dtype=torch.float32, device=dev)
         nd = ctx.num_decode
         if nd > 0:
-            K.hgrn2_scan(proj, self.q_col, self.v_col, f, state, o, ctx.seq_starts[:nd + 1], ctx.state_slots[:nd],
+            K.hgrn2_scan(proj, self.q_col, self.v_col, f, k, state, o, ctx.seq_starts[:nd + 1], ctx.state_slots[:nd],
                          self.nh, self.dim, self.vdim)
         if ctx.num_seqs > nd:
             tiles, num_tiles = ctx.row_tiles(K.PREFILL_TILE_ROWS)
-            K.hgrn2_chunked(proj, self.q_col, self.v_col, f, state, o, ctx.seq_starts, ctx.state_slots, tiles, num_tiles,
+            K.hgrn2_chunked(proj, self.q_col, self.v_col, f, k, state, o, ctx.seq_starts, ctx.state_slots, tiles, num_tiles,
                             nd, self.nh, self.dim, self.vdim)
         normed = torch.empty((n, self.nv), dtype=self.rt.dtype, device=dev)
         K.head_norm_gate(o, None, 0, self.w_norm, self.norm_eps, self.nh, self.vdim, normed)
@@ -96,10 +97,11 @@ class Hgrn2(Mixer):
         program.keep(state, self.b_f, self.lower, self.w_norm)
         proj = emit_linear(program, program.x, N, self.w_in, rt.dtype, None, False, "hgrn2.proj", "hgrn2.in").tensor()
         f = emit_linear(program, program.x, N, self.w_f, torch.float32, None, False, "hgrn2.f", "hgrn2.gate").tensor()
-        program.op("core", "ia_hgrn2_gates", [proj, act, self.row, self.q_col, f, self.nq, self.b_f, self.lower, N,
+        k = program.buffer("hgrn2.k", T * self.nq * 4)
+        program.op("core", "ia_hgrn2_gates", [proj, act, self.row, self.q_col, f, k, self.nq, self.b_f, self.lower, N,
                                               self.nq, STREAM])
         o = program.buffer("hgrn2.o", T * self.nv * 4)
-        program.op("core", "ia_hgrn2_scan", [proj, act, self.row, self.q_col, self.v_col, f, self.nq, state,
+        program.op("core", "ia_hgrn2_scan", [proj, act, self.row, self.q_col, self.v_col, f, k, self.nq, state,
                                              int(state.stride(0)), o, program.seq_starts, program.state_slots,
                                              program.ND, self.nh, self.dim, self.vdim, STREAM],
                    Guard.between(program.ND, 1))
@@ -108,7 +110,7 @@ class Hgrn2(Mixer):
         records = program.buffer("hgrn2.records", most * floats * 4)
         decay = program.buffer("hgrn2.decay", most * self.nq * 4)
         tiles, num_tiles = program.row_tiles(K.PREFILL_TILE_ROWS)
-        program.op("core", "ia_hgrn2_chunked", [proj, act, self.row, self.q_col, self.v_col, f, self.nq, state,
+        program.op("core", "ia_hgrn2_chunked", [proj, act, self.row, self.q_col, self.v_col, f, k, self.nq, state,
                                                 int(state.stride(0)), o, program.seq_starts, program.state_slots, tiles,
                                                 num_tiles, program.ND, N, records, floats, decay, self.nh, self.dim,
                                                 self.vdim, STREAM], Guard.between(program.NP, 1))

@@ -61,8 +61,10 @@ def _shape_fits(found: tuple, wanted: tuple) -> bool:
     return len(found) == len(wanted) and all(w == -1 or int(f) == int(w) for f, w in zip(found, wanted))
 
 
-def check_against(expected: Dict[str, WeightSpec], found: Dict[str, tuple], where: str) -> Dict[str, str]:
-    """Compare names and shapes; returns expected name -> name to read it from."""
+def check_against(expected: Dict[str, WeightSpec], found: Dict[str, tuple], where: str,
+                  ignored: tuple = ()) -> Dict[str, str]:
+    """Compare names and shapes; returns expected name -> name to read it from.  ``ignored``: patterns of names
+    that the file may hold without a part that reads them (a model's own, beside IGNORED_TENSORS)."""
     missing, wrong = [], []
     source: Dict[str, str] = {}
     used = set()
@@ -78,7 +80,7 @@ def check_against(expected: Dict[str, WeightSpec], found: Dict[str, tuple], wher
             wrong.append(f"{name}: expected {list(spec.shape)} got {list(found[src])}")
         source[name] = src
     unexpected = sorted(n for n in found if n not in used and n not in expected
-                        and not any(fnmatch.fnmatch(n, pat) for pat in IGNORED_TENSORS))
+                        and not any(fnmatch.fnmatch(n, pat) for pat in IGNORED_TENSORS + tuple(ignored)))
     if missing or unexpected or wrong:
         raise WeightError(where, sorted(missing), unexpected, wrong)
     return source
@@ -119,7 +121,8 @@ def load_weights(model, model_dir: str) -> None:
     rt: Runtime = model.rt
     expected = model.expected_weights()
     entries: Dict[str, TensorEntry] = open_model_tensors(model_dir)
-    source = check_against(expected, {n: e.shape for n, e in entries.items()}, model_dir)
+    source = check_against(expected, {n: e.shape for n, e in entries.items()}, model_dir,
+                           tuple(getattr(model.spec, "ignored_tensors", ())))
     # a tied head shares the embedding's buffer: one key for both
     keys = {name: (source[name], spec.follows_compute_dtype) for name, spec in expected.items()}
     model.load_weights(LazyTensors(keys, lambda name, key: _convert(entries[key[0]].read(), expected[name], rt)))

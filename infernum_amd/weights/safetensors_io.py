@@ -130,5 +130,6 @@ def write_safetensors(path: str, tensors: Iterable[Tuple[str, torch.Tensor]]) ->
         f.write(blob)
         for t in staged:
             if t.numel():
-                f.write(t.view(torch.uint8).numpy().tobytes() if t.dtype != torch.bool else t.numpy().tobytes())
+                flat = t.reshape(-1)            # a tensor without dimensions (one number) has no bytes to view
+                f.write(flat.view(torch.uint8).numpy().tobytes() if t.dtype != torch.bool else flat.numpy().tobytes())
     os.replace(tmp, path)

@@ -98,7 +98,8 @@ def attention_mixer(a: torch.Tensor, w: Mapping[str, torch.Tensor], p: str, m: M
         q, k = rotate(q, ang, rot["dims"], "half"), rotate(k, ang, rot["dims"], "half")
     q, k = _r(unit_rms(q, eps), round_to), _r(unit_rms(k, eps), round_to)
     mask = m.get("mask")
-    size, pool = (int(mask["size"]), int(mask["pool"])) if mask else (T + 1, T + 1)
+    size = int(mask["size"]) if mask else T + 1                  # no mask: every earlier key
+    pool = int(mask["pool"]) if mask and mask.get("pool") else T + 1          # no blocks: what leaves the window is gone
     B = T // pool
     out = torch.zeros((T, H, dv), dtype=F64)
     for h in range(H):
@@ -237,3 +238,64 @@ def forward(cfg: Mapping, w: Mapping[str, torch.Tensor], tokens, round_to=None, 
         if streams is not None:
             streams.append(x.clone())
     return _r(unit_rms(x, eps) * w["final.norm"], round_to) @ w["head"].T
+
+
+# ---------------------------------------------------------------------------------------------- weights for tests
+def tensor_shapes(cfg: Mapping) -> Dict[str, Tuple[int, ...]]:
+    """Names and shapes of a model's tensors."""
+    V, W = cfg["vocab"], cfg["width"]
+    side = cfg.get("token_side")
+    out: Dict[str, Tuple[int, ...]] = {"embed": (V, W)}
+    if side:
+        out["side.embed"] = (V, int(side["dim"]) * len(cfg["layers"]))
+    for i, layer in enumerate(cfg["layers"]):
+        p, m = f"l{i}.", layer["mixer"]
+        out[p + "norm1"] = ()
+        if layer["type"] == "attention":
+            H, G, d, dv = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
+            out.update({p + "mix.q": (H * d, W), p + "mix.q.b": (H * d,), p + "mix.k": (G * d, W), p + "mix.k.b": (G * d,),
+                        p + "mix.v": (G * dv, W), p + "mix.v.b": (G * dv,), p + "mix.o": (W, H * dv)})
+        elif layer["type"] == "latent_attention":
+            H, d, dr, dv, rk, rq = m["heads"], m["dim"], m["rot_dim"], m["vdim"], m["kv_rank"], m["q_rank"]
+            out.update({p + "mix.dq": (rq, W), p + "mix.dq.norm": (rq,), p + "mix.uq": (H * (d + dr), rq),
+                        p + "mix.dkv": (rk + dr, W), p + "mix.dkv.norm": (rk,), p + "mix.uk": (H * d, rk),
+                        p + "mix.uv": (H * dv, rk), p + "mix.sink": (H,), p + "mix.o": (W, H * dv)})
+        else:
+            H, d, dv = m["heads"], m["dim"], m["vdim"]
+            out.update({p + "mix.q": (H * d, W), p + "mix.f": (H * d, W), p + "mix.f.b": (H * d,),
+                        p + "mix.lower": (H * d,), p + "mix.v": (H * dv, W), p + "mix.norm": (dv,), p + "mix.o": (W, H * dv)})
+        if layer.get("mlp") is not None:
+            ff = layer["mlp"]["ff"]
+            out.update({p + "norm2": (), p + "mlp.gate": (ff, W), p + "mlp.up": (ff, W), p + "mlp.down": (W, ff)})
+        if side:
+            out.update({p + "side.gate": (int(side["dim"]), W), p + "side.proj": (W, int(side["dim"])), p + "side.norm": (W,)})
+    out["final.norm"] = ()
+    out["head"] = (V, W)
+    return out
+
+
+def random_weights(cfg: Mapping, seed: int = 0, store: torch.dtype = torch.bfloat16) -> Dict[str, torch.Tensor]:
+    """Weights of a size that keeps every branch of order one; rounded to ``store``."""
+    g = torch.Generator().manual_seed(seed)
+    out = {}
+    for name, shape in tensor_shapes(cfg).items():
+        last = name.rsplit(".", 1)[-1]
+        rnd = lambda: torch.randn(shape, generator=g)                               # noqa: E731
+        if "norm" in last:
+            t = 1.0 + 0.2 * rnd()
+        elif name.endswith("f.b"):
+            t = -1.0 + 4.0 * torch.rand(shape, generator=g)          # gates between forgetting fast and slowly
+        elif last == "lower":
+            t = 0.9 * torch.rand(shape, generator=g)
+        elif last == "b":
+            t = 0.5 * rnd()
+        elif last == "sink":
+            t = rnd()
+        elif name in ("embed", "side.embed"):
+            t = rnd()
+        elif last in ("q", "k", "uq", "uk") and "mix" in name:
+            t = 2.0 * rnd() / math.sqrt(shape[-1])                   # scores of some size, so that the masks matter
+        else:
+            t = rnd() / math.sqrt(shape[-1])
+        out[name] = t.to(store)
+    return out
