@@ -574,6 +574,65 @@ def malinex_active_params(size: dict) -> int:
     return (n // 4) * attention + (n - n // 4) * gla + (n // 2) * dense + (n - n // 2) * moe + n * gates + size["vocab"] * W
 
 
+# ---- the Sikazen design beside the Llama decoder at equal sizes -------------------------------------------------
+# Four layers of one width that run twice (a loop over all of them: eight layer runs, the embedding's rows added before
+# the second pass): attention over a window of keys and pooled blocks before it (heads of 128 over 4 key/value heads,
+# blocks of 64), latent attention with a query latent and sinks (a latent head of 32 + 224), HGRN2 (heads of 128 x 128),
+# and the first kind again; every layer with the twin's gated feed-forward beside its mixer, and a token input of 256
+# values a layer.  The Llama twin has eight layers of the same width, vocabulary, heads and feed-forward.
+SIKAZEN_SIZES = {
+    "2k": dict(width=2048, runs=8, vocab=32000, ff=5504, heads=16, kv_heads=4, dim=128, window=1024, pool=64,
+               lat_dim=64, lat_rot=32, lat_rank=224, q_rank=768, side=256),
+    "4k": dict(width=4096, runs=8, vocab=32000, ff=9600, heads=32, kv_heads=8, dim=128, window=2048, pool=64,
+               lat_dim=64, lat_rot=32, lat_rank=224, q_rank=1536, side=256),
+}
+
+
+def sikazen_configs(size: dict):
+    from infernum_amd.config import LlamaConfig
+    from infernum_amd.config.sikazen import SikazenConfig
+    d = size["dim"]
+    attention = {"heads": size["heads"], "kv_heads": size["kv_heads"], "dim": d, "vdim": d, "scale": d ** -0.5 * 4,
+                 "mask": {"size": size["window"], "pool": size["pool"]},
+                 "rot": {"base": 10000.0, "dims": d, "scaling": {"factor": 4.0}}}
+    latent = {"heads": size["heads"], "dim": size["lat_dim"], "rot_dim": size["lat_rot"], "vdim": size["lat_dim"],
+              "kv_rank": size["lat_rank"], "q_rank": size["q_rank"], "scale": (size["lat_dim"] + size["lat_rot"]) ** -0.5,
+              "rot": {"base": 10000.0, "dims": size["lat_rot"]}}
+    hgrn2 = {"heads": size["heads"], "dim": d, "vdim": d}
+    mlp = {"kind": "dense", "ff": size["ff"]}
+    kinds = [("attention", attention), ("latent_attention", latent), ("hgrn2", hgrn2), ("attention", attention)]
+    sik = SikazenConfig.from_dict({
+        "architecture": "Sikazen", "vocab": size["vocab"], "width": size["width"], "embedding": {"scale": 1.0},
+        "norm": {"eps": 1e-6}, "token_side": {"dim": size["side"]},
+        "loop": {"start": 0, "stop": len(kinds), "times": size["runs"] // len(kinds)},
+        "layers": [{"type": k, "mixer": m, "mlp": mlp} for k, m in kinds]})
+    llama = LlamaConfig.from_dict(dict(
+        model_type="llama", num_hidden_layers=size["runs"], hidden_size=size["width"],
+        num_attention_heads=size["heads"], num_key_value_heads=size["kv_heads"], intermediate_size=size["ff"],
+        vocab_size=size["vocab"], rope_theta=10000.0, rms_norm_eps=1e-6, tie_word_embeddings=True,
+        max_position_embeddings=8192))
+    return sik, llama
+
+
+def sikazen_active_params(size: dict) -> int:
+    """Weights that a token multiplies with in the Sikazen model of these sizes (every layer run and the head)."""
+    W, d, H = size["width"], size["dim"], size["heads"]
+    attention = W * (H + 2 * size["kv_heads"]) * d + H * d * W
+    lat_q = size["lat_dim"] + size["lat_rot"]
+    latent = (W * (size["q_rank"] + size["lat_rank"] + size["lat_rot"]) + size["q_rank"] * H * lat_q
+              + H * size["lat_rank"] * 2 * size["lat_dim"] + H * size["lat_dim"] * W)
+    hgrn2 = W * 3 * H * d + H * d * W
+    side = 2 * W * size["side"]
+    per_pass = 2 * attention + latent + hgrn2 + 4 * (3 * W * size["ff"] + side)
+    return (size["runs"] // 4) * per_pass + size["vocab"] * W
+
+
+def sikazen_bench(a) -> int:
+    batches = [int(b) for b in a.sikazen_batches.split(",") if b]
+    return beside_llama_bench(a, "Sikazen", [(n, SIKAZEN_SIZES[n]) for n in a.sikazen.split(",")], sikazen_configs,
+                              sikazen_active_params, batches)
+
+
 def malinex_bench(a) -> int:
     batches = [int(b) for b in a.malinex_batches.split(",") if b]
     return beside_llama_bench(a, "Malinex", [(n, MALINEX_SIZES[n]) for n in a.malinex.split(",")], malinex_configs,
@@ -691,6 +750,11 @@ def main() -> int:
                     help="the Malinex design (gated linear attention, attention with sigmoid weights, routed experts) beside "
                          "the Llama decoder at equal sizes: names of " + ", ".join(MALINEX_SIZES) + " with commas")
     ap.add_argument("--malinex-batches", default="8,64", help="decode batches of --malinex")
+    ap.add_argument("--sikazen", default="", metavar="SIZES",
+                    help="the Sikazen design (attention over a window and pooled blocks, latent attention with sinks, HGRN2, "
+                         "parallel sublayers) beside the Llama decoder at equal sizes: names of "
+                         + ", ".join(SIKAZEN_SIZES) + " with commas")
+    ap.add_argument("--sikazen-batches", default="8,64", help="decode batches of --sikazen")
     a = ap.parse_args()
     if a.gpus != 1:
         print(f"bench.py measures one GPU: this engine has no multi-GPU path (asked for --gpus {a.gpus})")
@@ -700,6 +764,8 @@ def main() -> int:
         return nesilorn_bench(a)
     if a.malinex:
         return malinex_bench(a)
+    if a.sikazen:
+        return sikazen_bench(a)
     if a.rogizen:
         return rogizen_bench(a)
     if a.decode_kernels:

@@ -64,6 +64,8 @@ DEFAULT_HEAD_DIMS = (16, 32, 48, 64, 80, 96, 112, 128, 160, 192, 256)
 SUPPORTED_HEAD_DIMS = tuple(range(16, 257, 16))
 # (key size, value size) pairs whose sigmoid-attention library `build_all` compiles ahead of time.
 DEFAULT_SIGATTN_SIZES = ((16, 32), (32, 64), (48, 16), (64, 64), (64, 128), (96, 32), (128, 32), (128, 64), (128, 128))
+# (key size, value size) pairs whose window-and-blocks attention library `build_all` compiles ahead of time.
+DEFAULT_WPA_SIZES = ((16, 16), (16, 32), (32, 16), (48, 16), (64, 64), (128, 128))
 
 
 class BuildError(RuntimeError):
@@ -140,7 +142,8 @@ def _fingerprint(sources: Sequence[str], defines: Sequence[str], host: bool = Fa
 
 
 def library_plan(name: str) -> Dict:
-    """Sources and defines of a library by its name ('core', 'attn_d<D>', 'sigattn_d<D>_v<V>', 'host' or 'blaslt')."""
+    """Sources and defines of a library by its name ('core', 'attn_d<D>', 'sigattn_d<D>_v<V>', 'wpa_d<D>_v<V>', 'host'
+    or 'blaslt')."""
     if name == "host":
         return {"sources": _existing(HOST_SOURCES), "defines": [], "host": True}
     if name == "blaslt":
@@ -165,6 +168,12 @@ def library_plan(name: str) -> Dict:
             raise BuildError(f"no MFMA sigmoid-attention kernel named {name!r}: key and value sizes are multiples of "
                              "16 up to 256")
         return {"sources": ["sigmoid_attention_mfma.hip"], "defines": [f"-DSA_DIM={int(d)}", f"-DSA_VDIM={int(v)}"]}
+    if name.startswith("wpa_d"):
+        d, _, v = name[len("wpa_d"):].partition("_v")
+        if not (d.isdigit() and v.isdigit() and int(d) in SUPPORTED_HEAD_DIMS and int(v) in SUPPORTED_HEAD_DIMS):
+            raise BuildError(f"no MFMA window-and-blocks attention kernel named {name!r}: key and value sizes are "
+                             "multiples of 16 up to 256")
+        return {"sources": ["window_pool_attention_mfma.hip"], "defines": [f"-DWP_DIM={int(d)}", f"-DWP_VDIM={int(v)}"]}
     raise BuildError(f"unknown library {name!r}")
 
 
@@ -273,6 +282,8 @@ def build_all(head_dims: Sequence[int] = DEFAULT_HEAD_DIMS) -> List[str]:
         names += [f"attn_d{d}" for d in head_dims]
     if os.path.isfile(os.path.join(CSRC_DIR, "sigmoid_attention_mfma.hip")):
         names += [f"sigattn_d{d}_v{v}" for d, v in DEFAULT_SIGATTN_SIZES]
+    if os.path.isfile(os.path.join(CSRC_DIR, "window_pool_attention_mfma.hip")):
+        names += [f"wpa_d{d}_v{v}" for d, v in DEFAULT_WPA_SIZES]
     workers = max(1, min(4, int(os.environ.get("MAX_JOBS", "8"))))
     with concurrent.futures.ThreadPoolExecutor(workers) as ex:
         return list(ex.map(compile_library, names))

@@ -17,7 +17,8 @@
 //   ia_rms_rows        y = x / sqrt(mean(x^2) + eps) * w over C values of every row (w nullable).
 //   ia_gelu_mul_rows   y[n, j] = gelu_tanh(u[n, j]) * table[ids[n], col0 + j].
 //
-// Token pages: keys [num_pages, nkv, page_size, d], values [num_pages, nkv, page_size, dv].  Pooled pages:
+// Token pages: keys [num_pages, nkv, page_size, d], values transposed within the page, [num_pages, nkv, dv, page_size]
+// (what the matrix-core kernels of window_pool_attention_mfma.hip read 8 bytes at a time).  Pooled pages:
 // [num_pages, nkv, E, d] and [.., E, dv] with E = (page_size - 1) / P + 1 entries a page: block b lies in the page of
 // its last position t = b P + P - 1, at entry (t % page_size) / P.  The token pages and the pooled pages have block
 // tables of their own (the token pages may be given back once the window and the open block have passed them).
@@ -41,6 +42,7 @@ __global__ __launch_bounds__(64) void wpa_prepare_kernel(
   for (int i = lane; i < size; i += 64) x[i] = to_float(s[i]) + (bias ? bias[col + i] : 0.f);
   __syncthreads();
   T* dst;
+  size_t step = 1;               // from a value to the next where it is written
   if (!is_v) {
     const int half = rot >> 1, pos = positions[n];
     for (int i = lane; i < half; i += 64) {
@@ -66,9 +68,12 @@ __global__ __launch_bounds__(64) void wpa_prepare_kernel(
     const int slot = slots[n], page = slot / ps, off = slot - page * ps;
     if ((unsigned)page >= (unsigned)num_pages) return;
     if (is_k) dst = k_pages + (((size_t)page * nkv + (head - nh)) * ps + off) * d;
-    else dst = v_pages + (((size_t)page * nkv + (head - nh - nkv)) * ps + off) * dv;
+    else {
+      dst = v_pages + ((size_t)page * nkv + (head - nh - nkv)) * dv * ps + off;
+      step = (size_t)ps;
+    }
   }
-  for (int i = lane; i < size; i += 64) dst[i] = from_float<T>(x[i]);
+  for (int i = lane; i < size; i += 64) dst[i * step] = from_float<T>(x[i]);
 }
 
 extern "C" int ia_wpa_prepare(const void* src, int src_stride, const float* bias, void* q_out, int q_stride, int dtype,
@@ -125,9 +130,9 @@ __global__ __launch_bounds__(64) void wpa_pool_kernel(const T* __restrict__ k_pa
     for (int j = pos - P + 1; j <= pos; ++j) {          // in the order of the positions
       const int page = bt[j / ps];
       if ((unsigned)page >= (unsigned)num_pages) { bad = true; break; }
-      const size_t row = ((size_t)page * nkv + g) * ps + (j % ps);
-      if (i < d) ak += to_float(k_pages[row * d + i]);
-      if (i < dv) av += to_float(v_pages[row * dv + i]);
+      const size_t head_page = (size_t)page * nkv + g;
+      if (i < d) ak += to_float(k_pages[(head_page * ps + (j % ps)) * d + i]);
+      if (i < dv) av += to_float(v_pages[(head_page * dv + i) * ps + (j % ps)]);
     }
     if (bad) ak = av = __uint_as_float(0x7fc00000u);     // a key of the block has no page: poison, never a stray read
     if (i < d) pk[i] = from_float<T>(ak * inv);
@@ -163,10 +168,11 @@ extern "C" int ia_wpa_pool(const void* k_pages, const void* v_pages, void* pk_pa
 
 // One stretch of up to 64 keys (or blocks): lane `lane` holds the key at row `row` of its pool when `valid`;
 // `ok` false: the key is needed and has no page.  Updates the running maximum, denominator and sums.
+// ``row``: the key's row in its pool; ``vat``: where the key's first value stands, ``vstep`` from a value to the next.
 template <typename T>
 __device__ __forceinline__ void wpa_round(const float* qs, const T* __restrict__ kp, const T* __restrict__ vp, bool valid,
-                                          bool ok, size_t row, int cnt, int d, int dv, float scale, float& m, float& l,
-                                          float* acc, float* ps_, size_t* rs_) {
+                                          bool ok, size_t row, size_t vat, size_t vstep, int cnt, int d, int dv,
+                                          float scale, float& m, float& l, float* acc, float* ps_, size_t* rs_) {
   const int lane = threadIdx.x;
   float sc = -INFINITY;
   if (valid) {
@@ -186,15 +192,15 @@ __device__ __forceinline__ void wpa_round(const float* qs, const T* __restrict__
 #pragma unroll
   for (int c = 0; c < WPA_MAX_D / 64; ++c) acc[c] *= corr;
   ps_[lane] = p;
-  rs_[lane] = ok ? row : 0;
+  rs_[lane] = ok ? vat : 0;
   __syncthreads();
   for (int jj = 0; jj < cnt; ++jj) {
-    const T* vr = vp + rs_[jj] * dv;
+    const T* vr = vp + rs_[jj];
     const float pj = ps_[jj];
 #pragma unroll
     for (int c = 0; c < WPA_MAX_D / 64; ++c) {
       const int dim = lane + 64 * c;
-      if (dim < dv) acc[c] = fmaf(pj, to_float(vr[dim]), acc[c]);
+      if (dim < dv) acc[c] = fmaf(pj, to_float(vr[(size_t)dim * vstep]), acc[c]);
     }
   }
   __syncthreads();
@@ -237,8 +243,8 @@ __global__ __launch_bounds__(64) void wpa_attention_kernel(
         ok = (unsigned)page < (unsigned)num_pool_pages;
         if (ok) row = ((size_t)page * nkv + g) * E + (t % ps) / P;
       }
-      wpa_round<T>(qs, pk_pages, pv_pages, valid, ok, row, (nb - b0) < 64 ? (nb - b0) : 64, d, dv, scale, m, l, acc, ps_,
-                   rs_);
+      wpa_round<T>(qs, pk_pages, pv_pages, valid, ok, row, row * dv, 1, (nb - b0) < 64 ? (nb - b0) : 64, d, dv, scale, m,
+                   l, acc, ps_, rs_);
     }
   }
   // the window's keys
@@ -249,14 +255,17 @@ __global__ __launch_bounds__(64) void wpa_attention_kernel(
       const int j = j0 + lane;
       const bool valid = j <= pos;
       bool ok = false;
-      size_t row = 0;
+      size_t row = 0, vat = 0;
       if (valid) {
         const int page = bt[j / ps];
         ok = (unsigned)page < (unsigned)num_pages;
-        if (ok) row = ((size_t)page * nkv + g) * ps + (j % ps);
+        if (ok) {
+          row = ((size_t)page * nkv + g) * ps + (j % ps);
+          vat = ((size_t)page * nkv + g) * dv * ps + (j % ps);
+        }
       }
-      wpa_round<T>(qs, k_pages, v_pages, valid, ok, row, (pos - j0 + 1) < 64 ? (pos - j0 + 1) : 64, d, dv, scale, m, l,
-                   acc, ps_, rs_);
+      wpa_round<T>(qs, k_pages, v_pages, valid, ok, row, vat, (size_t)ps, (pos - j0 + 1) < 64 ? (pos - j0 + 1) : 64, d, dv,
+                   scale, m, l, acc, ps_, rs_);
     }
   }
   if (sinks) {

@@ -1453,7 +1453,7 @@ def wpa_prepare(proj: torch.Tensor, bias: Optional[torch.Tensor], q_out: torch.T
     """From rows [nh q heads of d | nkv k heads of d | nkv v heads of dv] (+ ``bias`` fp32): rotation of the first
     ``rot`` values of every q and k head (value i with i + rot/2), then (``unit_norm``) every q and k head divided by
     its root mean square; queries to ``q_out`` [N, nh d], keys to ``k_pages`` [pages, nkv, page, d] and values to
-    ``v_pages`` [pages, nkv, page, dv] at ``slots``."""
+    ``v_pages`` (transposed within a page: [pages, nkv, dv, page]) at ``slots``."""
     N = proj.shape[0]
     row = (nh + nkv) * d + nkv * dv
     _rows(proj, row, "wpa_prepare rows")
@@ -1467,8 +1467,8 @@ def wpa_prepare(proj: torch.Tensor, bias: Optional[torch.Tensor], q_out: torch.T
               and freq.numel() == rot // 2 and rot % 2 == 0 and rot <= d, "wpa_prepare: rot/2 frequencies, rot even, <= d")
     num_pages, ps = k_pages.shape[0], k_pages.shape[2]
     _need(k_pages.dtype == proj.dtype and v_pages.dtype == proj.dtype and k_pages.is_contiguous() and v_pages.is_contiguous()
-          and tuple(k_pages.shape) == (num_pages, nkv, ps, d) and tuple(v_pages.shape) == (num_pages, nkv, ps, dv),
-          "wpa_prepare: key pages [num_pages, nkv, page_size, d], value pages [num_pages, nkv, page_size, dv]")
+          and tuple(k_pages.shape) == (num_pages, nkv, ps, d) and tuple(v_pages.shape) == (num_pages, nkv, dv, ps),
+          "wpa_prepare: key pages [num_pages, nkv, page_size, d], value pages [num_pages, nkv, dv, page_size]")
     _ok(_core().ia_wpa_prepare(_p(proj), int(proj.stride(0)), _p(bias), _p(q_out), int(q_out.stride(0)),
                                DTYPE_CODE[proj.dtype], _p(positions), _p(slots), _p(freq if rot else None),
                                1 if (rot and freq.dtype == torch.float64) else 0, int(rot), int(bool(unit_norm)),
@@ -1484,7 +1484,8 @@ def wpa_pool(k_pages: torch.Tensor, v_pages: torch.Tensor, pk_pages: torch.Tenso
     and values, read from the token pages, into the pooled pages ([pages, nkv, wpa_pool_entries, d | dv])."""
     N = positions.numel()
     num_pages, nkv, ps, d = k_pages.shape
-    dv = v_pages.shape[3]
+    dv = v_pages.shape[2]
+    _need(tuple(v_pages.shape) == (num_pages, nkv, dv, ps), "wpa_pool: value pages [num_pages, nkv, dv, page_size]")
     E = wpa_pool_entries(ps, pool)
     _need(tuple(pk_pages.shape[1:]) == (nkv, E, d) and tuple(pv_pages.shape[1:]) == (nkv, E, dv)
           and pk_pages.dtype == k_pages.dtype == v_pages.dtype == pv_pages.dtype and pk_pages.is_contiguous()
@@ -1508,11 +1509,11 @@ def wpa_attention(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
     over both, ``sinks`` fp32 [nh] in its denominator.  ``out`` [N, nh dv]."""
     N = out.shape[0]
     num_pages, _, ps, d = k_pages.shape
-    dv = v_pages.shape[3]
+    dv = v_pages.shape[2]
     _rows(q, nh * d, "wpa_attention q")
     _need(out.is_cuda and out.is_contiguous() and tuple(out.shape) == (N, nh * dv) and q.shape[0] == N
           and q.dtype == out.dtype == k_pages.dtype == v_pages.dtype and q.dtype in DTYPE_CODE
-          and tuple(k_pages.shape) == (num_pages, nkv, ps, d) and tuple(v_pages.shape) == (num_pages, nkv, ps, dv)
+          and tuple(k_pages.shape) == (num_pages, nkv, ps, d) and tuple(v_pages.shape) == (num_pages, nkv, dv, ps)
           and k_pages.is_contiguous() and v_pages.is_contiguous(), "wpa_attention: q, pages and out [N, nh dv] of one dtype")
     _f32(sinks, nh, "wpa_attention sinks")
     _i32(token_seq, N, "wpa_attention token_seq")
@@ -1531,6 +1532,81 @@ def wpa_attention(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
                                  _p(bt_pool if pooled else None), bt_pool.shape[1] if pooled else 0, N, nh, nkv, d, dv, ps,
                                  num_pages, pk_pages.shape[0] if pooled else 0, ctypes.c_float(scale), int(window),
                                  int(pool) if pooled else 0, _stream()), "wpa_attention")
+    return out
+
+
+def wpa_mfma_available(d: int, dv: int) -> bool:
+    """Whether the matrix-core kernels of the window-and-blocks attention take these key and value sizes (their
+    library is built at its first use)."""
+    return d in _build.SUPPORTED_HEAD_DIMS and dv in _build.SUPPORTED_HEAD_DIMS
+
+
+def _wpa(d: int, dv: int) -> ctypes.CDLL:
+    return load_library(f"wpa_d{d}_v{dv}")
+
+
+def _wpa_check(q, k_pages, v_pages, pk_pages, pv_pages, out, sinks, bt_tokens, bt_pool, nh, nkv, window, pool, what):
+    num_pages, _, ps, d = k_pages.shape
+    dv = v_pages.shape[2]
+    N = out.shape[0]
+    _rows(q, nh * d, f"{what} q")
+    _need(q.dtype == torch.bfloat16 and out.dtype == torch.bfloat16 and k_pages.dtype == torch.bfloat16
+          and v_pages.dtype == torch.bfloat16 and out.is_cuda and out.is_contiguous() and tuple(out.shape) == (N, nh * dv)
+          and tuple(k_pages.shape) == (num_pages, nkv, ps, d) and tuple(v_pages.shape) == (num_pages, nkv, dv, ps)
+          and k_pages.is_contiguous() and v_pages.is_contiguous() and ps % 4 == 0 and q.stride(0) % 8 == 0,
+          f"{what}: bf16 q, key pages [num_pages, nkv, page_size, d], value pages [num_pages, nkv, dv, page_size] with "
+          "a page size in fours, out [N, nh dv]")
+    _f32(sinks, nh, f"{what} sinks")
+    _need(bt_tokens.dtype == torch.int32 and bt_tokens.dim() == 2 and bt_tokens.is_contiguous(), f"{what}: block tables")
+    pooled = pool > 0 and window > 0
+    if pooled:
+        E = wpa_pool_entries(ps, pool)
+        _need(pk_pages is not None and pv_pages is not None and bt_pool is not None and bt_pool.dtype == torch.int32
+              and bt_pool.is_contiguous() and pk_pages.dtype == q.dtype and pv_pages.dtype == q.dtype
+              and pk_pages.is_contiguous() and pv_pages.is_contiguous()
+              and tuple(pk_pages.shape[1:]) == (nkv, E, d) and tuple(pv_pages.shape[1:]) == (nkv, E, dv), f"{what}: pooled pages")
+    _dev(q, k_pages, v_pages, pk_pages, pv_pages, out, bt_tokens, bt_pool)
+    return pooled, ps, num_pages, d, dv
+
+
+def wpa_decode(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, pk_pages: Optional[torch.Tensor],
+               pv_pages: Optional[torch.Tensor], out: torch.Tensor, sinks: Optional[torch.Tensor],
+               positions: torch.Tensor, bt_tokens: torch.Tensor, bt_pool: Optional[torch.Tensor], nh: int, nkv: int,
+               scale: float, window: int, pool: int) -> torch.Tensor:
+    """:func:`wpa_attention` of B single tokens on the matrix cores, bf16: row b of q, out and the block tables is
+    token b at positions[b]."""
+    pooled, ps, num_pages, d, dv = _wpa_check(q, k_pages, v_pages, pk_pages, pv_pages, out, sinks, bt_tokens, bt_pool,
+                                              nh, nkv, window, pool, "wpa_decode")
+    B = out.shape[0]
+    _i32(positions, B, "wpa_decode positions")
+    _need(bt_tokens.shape[0] >= B and (not pooled or bt_pool.shape[0] >= B), "wpa_decode: a row of the block tables a token")
+    _ok(_wpa(d, dv).ia_wpa_decode(_p(q), int(q.stride(0)), _p(k_pages), _p(v_pages), _p(pk_pages if pooled else None),
+                                  _p(pv_pages if pooled else None), _p(out), _p(sinks), _p(positions), _p(bt_tokens),
+                                  bt_tokens.shape[1], _p(bt_pool if pooled else None), bt_pool.shape[1] if pooled else 0,
+                                  B, nh, nkv, ps, num_pages, pk_pages.shape[0] if pooled else 0, ctypes.c_float(scale),
+                                  int(window), int(pool) if pooled else 0, _stream()), "wpa_decode")
+    return out
+
+
+def wpa_prefill(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, pk_pages: Optional[torch.Tensor],
+                pv_pages: Optional[torch.Tensor], out: torch.Tensor, sinks: Optional[torch.Tensor],
+                seq_starts: torch.Tensor, seq_ctx: torch.Tensor, bt_tokens: torch.Tensor, bt_pool: Optional[torch.Tensor],
+                tiles: torch.Tensor, num_tiles: int, nh: int, nkv: int, scale: float, window: int, pool: int) -> torch.Tensor:
+    """:func:`wpa_attention` of portions of prompts on the matrix cores, bf16: request s brings rows seq_starts[s] ..
+    seq_starts[s+1]-1 after seq_ctx[s] cached tokens; tiles[i] = (s, first row of a block of PREFILL_TILE_ROWS)."""
+    pooled, ps, num_pages, d, dv = _wpa_check(q, k_pages, v_pages, pk_pages, pv_pages, out, sinks, bt_tokens, bt_pool,
+                                              nh, nkv, window, pool, "wpa_prefill")
+    B = bt_tokens.shape[0]
+    _i32(seq_starts, B + 1, "wpa_prefill seq_starts")
+    _i32(seq_ctx, B, "wpa_prefill seq_ctx")
+    _need(tiles.dtype == torch.int32 and tiles.is_cuda and tiles.is_contiguous() and tiles.numel() >= 2 * num_tiles,
+          "wpa_prefill: tiles int32 [num_tiles, 2]")
+    _ok(_wpa(d, dv).ia_wpa_prefill(_p(q), int(q.stride(0)), _p(k_pages), _p(v_pages), _p(pk_pages if pooled else None),
+                                   _p(pv_pages if pooled else None), _p(out), _p(sinks), _p(seq_starts), _p(seq_ctx),
+                                   _p(bt_tokens), bt_tokens.shape[1], _p(bt_pool if pooled else None),
+                                   bt_pool.shape[1] if pooled else 0, _p(tiles), int(num_tiles), nh, nkv, ps, num_pages,
+                                   pk_pages.shape[0] if pooled else 0, ctypes.c_float(scale), int(window),
+                                   int(pool) if pooled else 0, _stream()), "wpa_prefill")
     return out
 
 

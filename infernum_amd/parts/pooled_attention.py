@@ -13,7 +13,10 @@ earlier key is seen and nothing is pooled.
 What it keeps: the keys and values of the positions that the window or the open block still need (a ``window``
 group of pages whose reach is max(window, P): older pages go back to the pool), and the blocks' means in pages of
 a ``full`` group with one entry per P positions (``cached_companions``: a second cached thing with block tables of
-its own).  A block's means are made in the step that brings the block's last token, from the pages.
+its own).  A block's means are made in the step that brings the block's last token, from the pages.  In bfloat16,
+head sizes in multiples of 16 up to 256 run on the matrix cores (a kernel for single tokens, whose sixteen columns
+are the query heads of a key/value head, and one for portions of prompts); other sizes and the 32-bit path take the
+plain kernel, a wave a token and head.
 """
 from __future__ import annotations
 
@@ -67,13 +70,18 @@ class PooledWindowAttention(Mixer):
             raise ValueError("this mixer rotates halves, without a factor on sine and cosine")
         self.blocks = _PooledBlocks(self.nkv, self.d, self.dv, self.pool) if self.pool else None
         self.row = (self.nh + self.nkv) * self.d + self.nkv * self.dv
+        # bf16 steps run on the matrix cores where the head sizes have a library; otherwise, and in 32-bit, on the
+        # plain kernel (a wave a token and head)
+        self.use_mfma = (rt.kernels == "auto" and rt.dtype == torch.bfloat16 and rt.device.type == "cuda"
+                         and K.wpa_mfma_available(self.d, self.dv))
         self.w_qkv: Optional[torch.Tensor] = None
         self.b_qkv: Optional[torch.Tensor] = None
         self.w_o: Optional[torch.Tensor] = None
 
     # ---- what it needs ---------------------------------------------------
     def cache_spec(self) -> CacheSpec:
-        payload = (PageTensor("k", (self.nkv, self.d), token_axis=1), PageTensor("v", (self.nkv, self.dv), token_axis=1))
+        # values transposed within a page, as the second product of the matrix cores reads them
+        payload = (PageTensor("k", (self.nkv, self.d), token_axis=1), PageTensor("v", (self.nkv, self.dv), token_axis=2))
         if not self.window:
             return CacheSpec("full", payload=payload)
         # a page is needed while the window reaches it, or the block that is still open
@@ -81,6 +89,9 @@ class PooledWindowAttention(Mixer):
 
     def cached_companions(self) -> Dict[str, Any]:
         return {"blocks": self.blocks} if self.blocks is not None else {}
+
+    def step_needs(self) -> Dict[str, Any]:
+        return {"row_tiles": K.PREFILL_TILE_ROWS} if self.use_mfma else {}
 
     def weights(self) -> Dict[str, WeightSpec]:
         nh, nkv, d, dv, H = self.nh, self.nkv, self.d, self.dv, self.hidden_size
@@ -125,14 +136,25 @@ class PooledWindowAttention(Mixer):
             pk, pv, bt_pool = blocks.pages["pk"], blocks.pages["pv"], ctx.block_tables[blocks.group]
             K.wpa_pool(kp, vp, pk, pv, ctx.token_seq, ctx.positions, ctx.block_tables[g], bt_pool, self.pool)
         out = torch.empty((n, nh * dv), dtype=x.dtype, device=x.device)
-        K.wpa_attention(q, kp, vp, pk, pv, out, None, ctx.token_seq, ctx.positions, ctx.block_tables[g], bt_pool, nh, nkv,
-                        self.scale, self.window, self.pool)
+        bt = ctx.block_tables[g]
+        if self.use_mfma and kp.shape[2] % 4 == 0:
+            nd = ctx.num_decode
+            if nd > 0:
+                K.wpa_decode(q[:nd], kp, vp, pk, pv, out[:nd], None, ctx.positions[:nd], bt, bt_pool, nh, nkv, self.scale,
+                             self.window, self.pool)
+            if ctx.num_seqs > nd:
+                tiles, num_tiles = ctx.row_tiles(K.PREFILL_TILE_ROWS)
+                K.wpa_prefill(q, kp, vp, pk, pv, out, None, ctx.seq_starts, ctx.seq_ctx, bt, bt_pool, tiles, num_tiles,
+                              nh, nkv, self.scale, self.window, self.pool)
+        else:
+            K.wpa_attention(q, kp, vp, pk, pv, out, None, ctx.token_seq, ctx.positions, bt, bt_pool, nh, nkv, self.scale,
+                            self.window, self.pool)
         return linear(out, self.w_o, keep_split=True, kernels=self.rt.kernels)
 
     def native(self, program, view: CacheView) -> None:
         if type(self).forward is not PooledWindowAttention.forward:
             return super().native(program, view)
-        from ..engine.program import STREAM
+        from ..engine.program import STREAM, Guard
         nh, nkv, d, dv, rt = self.nh, self.nkv, self.d, self.dv, self.rt
         kp, vp, blocks = self._views(view)
         g = view.group
@@ -158,10 +180,21 @@ class PooledWindowAttention(Mixer):
                                                bt_pool, pool_cols, N, nkv, d, dv, ps, num_pages, pool_pages, self.pool,
                                                STREAM])
         out = program.buffer("wpa.out", T * nh * dv * ab)
-        program.op("core", "ia_wpa_attention", [q, nh * d, kp, vp, pk, pv, out, nh * dv, act, None, program.token_seq,
-                                                program.positions, bt, bt_cols, bt_pool, pool_cols, N, nh, nkv, d, dv,
-                                                ps, num_pages, pool_pages, float(self.scale), self.window, self.pool,
-                                                STREAM])
+        if self.use_mfma and ps % 4 == 0:
+            lib = K._wpa(d, dv)
+            tiles, num_tiles = program.row_tiles(K.PREFILL_TILE_ROWS)
+            program.op(lib, "ia_wpa_decode", [q, nh * d, kp, vp, pk, pv, out, None, program.positions, bt, bt_cols, bt_pool,
+                                              pool_cols, program.ND, nh, nkv, ps, num_pages, pool_pages, float(self.scale),
+                                              self.window, self.pool, STREAM], Guard.between(program.ND, 1))
+            program.op(lib, "ia_wpa_prefill", [q, nh * d, kp, vp, pk, pv, out, None, program.seq_starts, program.seq_ctx,
+                                               bt, bt_cols, bt_pool, pool_cols, tiles, num_tiles, nh, nkv, ps, num_pages,
+                                               pool_pages, float(self.scale), self.window, self.pool, STREAM],
+                       Guard.between(program.NP, 1))
+        else:
+            program.op("core", "ia_wpa_attention", [q, nh * d, kp, vp, pk, pv, out, nh * dv, act, None, program.token_seq,
+                                                    program.positions, bt, bt_cols, bt_pool, pool_cols, N, nh, nkv, d, dv,
+                                                    ps, num_pages, pool_pages, float(self.scale), self.window, self.pool,
+                                                    STREAM])
         program.pending = emit_linear(program, out, N, self.w_o, rt.dtype, None, True, "wpa.mix", "wpa.o")
 
 

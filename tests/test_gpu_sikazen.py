@@ -172,9 +172,9 @@ def _standing_out(dtype, T, star, size, pool, d=16, scale=3.0):
     as a member of a block (about 5 / pool), or not at all."""
     W = 8
     rt = runtime(dtype)
-    m = {"heads": 1, "kv_heads": 1, "dim": d, "vdim": 4, "scale": scale, "mask": {"size": size, "pool": pool}}
+    m = {"heads": 1, "kv_heads": 1, "dim": d, "vdim": 16, "scale": scale, "mask": {"size": size, "pool": pool}}
     w = {n: torch.zeros(s, dtype=torch.float64) for n, s in (("q", (d, W)), ("q.b", (d,)), ("k", (d, W)), ("k.b", (d,)),
-                                                             ("v", (4, W)), ("v.b", (4,)), ("o", (W, 4)))}
+                                                             ("v", (16, W)), ("v.b", (16,)), ("o", (W, 16)))}
     w["q"][0, 0] = 1.0          # q = (x0, 0, ...): with x0 = 1 a unit vector of length sqrt(d) along the first place
     w["k"][0, 1] = 1.0          # k = (x1, x2, 0, ...)
     w["k"][1, 2] = 1.0
@@ -311,6 +311,71 @@ def test_sinks_in_the_matrix_core_kernels_against_the_plain_kernel(nh, nkv, d, p
     assert rel_err(got, want.double().cpu()) <= 3e-2
 
 
+@pytest.mark.parametrize("nh,nkv,d,dv,ps,window,pool", [(4, 2, 16, 32, 4, 20, 6), (6, 2, 64, 64, 16, 72, 12), (20, 1, 32, 16, 8, 1, 1),
+                                                        (3, 3, 48, 16, 12, 0, 0), (4, 2, 16, 16, 16, 33, 16), (2, 1, 128, 128, 16, 7, 9),
+                                                        (17, 1, 16, 16, 4, 40, 5)])
+def test_window_and_blocks_on_the_matrix_cores_against_the_plain_kernel(nh, nkv, d, dv, ps, window, pool):
+    """Requests of unequal length with their pages in a shuffled order, NaN in every page that no request holds and in
+    the pages of keys that have left every window; single tokens at each request's last place, and portions that
+    begin anywhere, with and without sinks."""
+    from infernum_amd.kernels import api as K
+    g = torch.Generator().manual_seed(7)
+    lens, starts_at = [70, 33, 129, 16, 200], [0, 20, 64, 15, 131]
+    B, MB = len(lens), -(-max(lens) // ps)
+    num_pages = B * MB + 5
+    nan = float("nan")
+    kp = torch.full((num_pages, nkv, ps, d), nan)
+    vp = torch.full((num_pages, nkv, dv, ps), nan)
+    E = K.wpa_pool_entries(ps, pool) if pool else 1
+    pk, pv = torch.full((num_pages, nkv, E, d), nan), torch.full((num_pages, nkv, E, dv), nan)
+    perm = torch.randperm(num_pages, generator=g)
+    bt = torch.full((B, MB), -1, dtype=torch.int32)
+    btp = torch.full((B, MB), -1, dtype=torch.int32)
+    for b, n in enumerate(lens):
+        reach = max(window, pool) if window else n
+        for pg in range(-(-n // ps)):
+            page = int(perm[b * MB + pg])
+            btp[b, pg] = page
+            if (pg + 1) * ps > n - reach - ps:              # pages that some query of the tests below still needs
+                bt[b, pg] = page
+                kp[page] = torch.randn(nkv, ps, d, generator=g)
+                vp[page] = torch.randn(nkv, dv, ps, generator=g)
+            pk[page] = torch.randn(nkv, E, d, generator=g)
+            pv[page] = torch.randn(nkv, E, dv, generator=g)
+    dev = lambda t: t.to(torch.bfloat16).to(DEV) if t.dtype.is_floating_point else t.to(DEV)   # noqa: E731
+    kp, vp, pk, pv, bt, btp = map(dev, (kp, vp, pk, pv, bt, btp))
+    scale = 2.0 / math.sqrt(d)
+    for sinks in (None, (torch.randn(nh, generator=g) * 2 + 1).to(DEV)):
+        # single tokens
+        q = dev(torch.randn(B, nh * d, generator=g))
+        pos = torch.tensor([n - 1 for n in lens], dtype=torch.int32, device=DEV)
+        seq = torch.arange(B, dtype=torch.int32, device=DEV)
+        want, got = torch.empty((B, nh * dv), dtype=torch.bfloat16, device=DEV), torch.empty((B, nh * dv), dtype=torch.bfloat16, device=DEV)
+        K.wpa_attention(q, kp, vp, pk, pv, want, sinks, seq, pos, bt, btp, nh, nkv, scale, window, pool)
+        K.wpa_decode(q, kp, vp, pk, pv, got, sinks, pos, bt, btp, nh, nkv, scale, window, pool)
+        assert torch.isfinite(want.float()).all()
+        assert rel_err(got, want.double().cpu()) <= 3e-2
+        # portions: request b brings its rows from starts_at[b] on (what lies before is cached)
+        news = [n - s0 for n, s0 in zip(lens, starts_at)]
+        if window:          # the rows of a portion reach back from its first row: only portions whose keys have pages
+            news = [min(k, ps) for k in news]
+            first = [n - k for n, k in zip(lens, news)]
+        else:
+            first = starts_at
+        N = sum(news)
+        q = dev(torch.randn(N, nh * d, generator=g))
+        starts = torch.tensor([0] + list(torch.tensor(news).cumsum(0)), dtype=torch.int32, device=DEV)
+        ctx = torch.tensor(first, dtype=torch.int32, device=DEV)
+        seq = torch.cat([torch.full((k,), i, dtype=torch.int32) for i, k in enumerate(news)]).to(DEV)
+        pos = torch.cat([torch.arange(f, f + k, dtype=torch.int32) for f, k in zip(first, news)]).to(DEV)
+        tiles = torch.tensor([(s_, r) for s_, k in enumerate(news) for r in range(0, k, K.PREFILL_TILE_ROWS)], dtype=torch.int32).to(DEV)
+        want, got = torch.empty((N, nh * dv), dtype=torch.bfloat16, device=DEV), torch.empty((N, nh * dv), dtype=torch.bfloat16, device=DEV)
+        K.wpa_attention(q, kp, vp, pk, pv, want, sinks, seq, pos, bt, btp, nh, nkv, scale, window, pool)
+        K.wpa_prefill(q, kp, vp, pk, pv, got, sinks, starts, ctx, bt, btp, tiles, tiles.shape[0], nh, nkv, scale, window, pool)
+        assert torch.isfinite(want.float()).all()
+        assert rel_err(got, want.double().cpu()) <= 3e-2
+
+
 HGRN_CASES = [(SM.S1["layers"][2]["mixer"], 64, 150), (SM.S2["layers"][3]["mixer"], 100, 70), (SM.S3["layers"][1]["mixer"], 128, 131),
               (SM.S4["layers"][1]["mixer"], 80, 64)]
 
@@ -403,9 +468,9 @@ def models(tmp_path_factory):
                     rounded = PS.forward(cfg, w, t, round_to=to)
                     cost[to] = max(cost[to], (rounded - refs[r]).abs().max().item() / refs[r].pow(2).mean().sqrt().item())
         BF16_TOL[name] = max(TOL["bfloat16"], 3.0 * cost[torch.bfloat16])
-        # in 32-bit the plain model rounds what is stored between kernels and none of the sums inside them: five times
-        # that (a place where two logits' terms nearly cancel costs S3 2.6e-5 by it alone)
-        F32_TOL[name] = max(TOL["float32"], 5.0 * cost[torch.float32])
+        # in 32-bit the plain model rounds what is stored between kernels and none of the sums inside them: eight
+        # times that (a place that multiplies every rounding fifty times over costs S3 2.6e-5 by it alone)
+        F32_TOL[name] = max(TOL["float32"], 8.0 * cost[torch.float32])
         print(f"{name}: rounding alone costs {cost[torch.bfloat16]:.2e} (bfloat16) and {cost[torch.float32]:.2e} "
               f"(stored values in 32-bit) of the logits' RMS")
         out[name] = (d, cfg, w, reqs, ref, mreqs, mref)
@@ -504,7 +569,7 @@ def test_long_decoding(models, name, dtype):
     reqs, ref = _requests(cfg, w, (160,), 3)
     cost = max((PS.forward(cfg, w, t, round_to=torch.float32) - ref[r]).abs().max().item() / ref[r].pow(2).mean().sqrt().item()
                for r, t in reqs.items())
-    F32_TOL[name] = max(F32_TOL[name], 5.0 * cost)
+    F32_TOL[name] = max(F32_TOL[name], 8.0 * cost)
     eng = _engine(d, dtype, 16, 12)
     got = TT.run_steps(eng, TT.trace_tail_one_by_one(reqs, 150))
     _check(got, ref, dtype, f"{name} {dtype} long decoding", name)
