@@ -15,6 +15,7 @@
 //   ia_gated_group_norm    y * silu(z), then an RMS norm in equal parts of the row, times a weight
 //   ia_concat_cast         rows [cast(a) | b]: the operand of a product over two streams side by side
 //   ia_stream_add         the fp32 stream += a tensor or the partial sums of a split product
+//   ia_stream_add2        the same for two of them one after the other, leaving the rounded stream as well
 //   ia_add_bias, ia_softcap
 //
 // Everything between the loads and the stores is fp32: sums of squares, angles, decays, step sizes, the state.
@@ -1006,6 +1007,96 @@ extern "C" int ia_stream_add(float* h, const void* delta, int code, int splits, 
   return IA_OK;
 }
 
+// h += a, then h += b (nullable), each a tensor or a stack of partial sums as in ia_stream_add, the additions in that
+// order; x (nullable) gets the new h in its own type: the two results of sublayers that ran side by side enter the
+// stream in one pass, which also leaves the rounded stream for whoever reads it next.  Four values a thread.
+__device__ __forceinline__ void sa2_load4(const void* p, int code, size_t i, float (&v)[4]) {
+  if (code == IA_F32) {
+    const float4 f = *reinterpret_cast<const float4*>(reinterpret_cast<const float*>(p) + i);
+    v[0] = f.x; v[1] = f.y; v[2] = f.z; v[3] = f.w;
+  } else {
+    const uint2 u = *reinterpret_cast<const uint2*>(reinterpret_cast<const uint16_t*>(p) + i);
+    v[0] = bf16_bits_to_float((uint16_t)(u.x & 0xffffu)); v[1] = bf16_bits_to_float((uint16_t)(u.x >> 16));
+    v[2] = bf16_bits_to_float((uint16_t)(u.y & 0xffffu)); v[3] = bf16_bits_to_float((uint16_t)(u.y >> 16));
+  }
+}
+__device__ __forceinline__ void sa2_sum4(const void* p, int code, int splits, size_t i, size_t n, float (&v)[4]) {
+  sa2_load4(p, code, i, v);
+  for (int k = 1; k < splits; ++k) {
+    float w[4];
+    sa2_load4(p, code, i + (size_t)k * n, w);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) v[e] += w[e];
+  }
+}
+template <bool VEC>
+__global__ __launch_bounds__(256) void stream_add2_kernel(float* __restrict__ h, const void* __restrict__ a, int a_code,
+                                                          int a_splits, const void* __restrict__ b, int b_code,
+                                                          int b_splits, void* __restrict__ x, int x_code, size_t n) {
+  const size_t stride = (size_t)gridDim.x * 256;
+  if (VEC) {
+    for (size_t i4 = (size_t)blockIdx.x * 256 + threadIdx.x; i4 < n / 4; i4 += stride) {
+      const size_t i = i4 * 4;
+      float hv[4], av[4];
+      sa2_load4(h, IA_F32, i, hv);
+      sa2_sum4(a, a_code, a_splits, i, n, av);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) hv[e] += av[e];
+      if (b) {
+        sa2_sum4(b, b_code, b_splits, i, n, av);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) hv[e] += av[e];
+      }
+      *reinterpret_cast<float4*>(h + i) = make_float4(hv[0], hv[1], hv[2], hv[3]);
+      if (x) {
+        if (x_code == IA_F32) {
+          *reinterpret_cast<float4*>(reinterpret_cast<float*>(x) + i) = make_float4(hv[0], hv[1], hv[2], hv[3]);
+        } else {
+          uint2 u;
+          u.x = (uint32_t)float_to_bf16_bits(hv[0]) | ((uint32_t)float_to_bf16_bits(hv[1]) << 16);
+          u.y = (uint32_t)float_to_bf16_bits(hv[2]) | ((uint32_t)float_to_bf16_bits(hv[3]) << 16);
+          *reinterpret_cast<uint2*>(reinterpret_cast<uint16_t*>(x) + i) = u;
+        }
+      }
+    }
+  } else {
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += stride) {
+      float v = h[i];
+      float t = load_as_float(a, a_code, i);
+      for (int k = 1; k < a_splits; ++k) t += load_as_float(a, a_code, i + (size_t)k * n);
+      v += t;
+      if (b) {
+        t = load_as_float(b, b_code, i);
+        for (int k = 1; k < b_splits; ++k) t += load_as_float(b, b_code, i + (size_t)k * n);
+        v += t;
+      }
+      h[i] = v;
+      if (x) {
+        if (x_code == IA_F32) reinterpret_cast<float*>(x)[i] = v;
+        else reinterpret_cast<uint16_t*>(x)[i] = float_to_bf16_bits(v);
+      }
+    }
+  }
+}
+
+extern "C" int ia_stream_add2(float* h, const void* a, int a_code, int a_splits, const void* b, int b_code, int b_splits,
+                              void* x, int x_code, int N, int H, hipStream_t stream) {
+  if (N == 0) return IA_OK;
+  if (!h || !a || N < 0 || H <= 0 || a_splits < 1 || (b && b_splits < 1)) return IA_ERR_BAD_ARG;
+  if ((a_code != IA_F32 && a_code != IA_BF16) || (b && b_code != IA_F32 && b_code != IA_BF16) ||
+      (x && x_code != IA_F32 && x_code != IA_BF16))
+    return IA_ERR_BAD_ARG;
+  const size_t n = (size_t)N * H;
+  const auto aligned = [](const void* p, size_t to) { return p == nullptr || (reinterpret_cast<uintptr_t>(p) % to) == 0; };
+  const bool vec = (n % 4) == 0 && aligned(h, 16) && aligned(a, 16) && aligned(b, 16) && aligned(x, 16);
+  const size_t items = vec ? n / 4 : n;
+  const unsigned grid = (unsigned)((items + 255) / 256 < 65536 ? (items + 255) / 256 : 65536);
+  if (vec) stream_add2_kernel<true><<<grid, 256, 0, stream>>>(h, a, a_code, a_splits, b, b_code, b_splits, x, x_code, n);
+  else stream_add2_kernel<false><<<grid, 256, 0, stream>>>(h, a, a_code, a_splits, b, b_code, b_splits, x, x_code, n);
+  IA_LAUNCH_CHECK();
+  return IA_OK;
+}
+
 // y [N, C] += bias (fp32 vector), rounded once
 template <typename T>
 __global__ __launch_bounds__(256) void add_bias_kernel(T* __restrict__ y, const float* __restrict__ bias, size_t n, int C) {
@@ -1053,5 +1144,6 @@ IA_OP(ia_ssd_chunked)
 IA_OP(ia_gated_group_norm)
 IA_OP(ia_concat_cast)
 IA_OP(ia_stream_add)
+IA_OP(ia_stream_add2)
 IA_OP(ia_add_bias)
 IA_OP(ia_softcap)

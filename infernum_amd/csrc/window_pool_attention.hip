@@ -102,16 +102,17 @@ extern "C" int ia_wpa_prepare(const void* src, int src_stride, const float* bias
   return IA_OK;
 }
 
-// grid (N, nkv), 64 threads.  A token that is not the last of its block leaves at once.
+// grid (N, nkv), 256 threads: a thread a value of the block's key or value, the block's positions added in their
+// order (the loads of several are in flight together).  A token that is not the last of its block leaves at once.
 template <typename T>
-__global__ __launch_bounds__(64) void wpa_pool_kernel(const T* __restrict__ k_pages, const T* __restrict__ v_pages,
-                                                      T* __restrict__ pk_pages, T* __restrict__ pv_pages,
-                                                      const int* __restrict__ token_seq,
-                                                      const int* __restrict__ positions, const int* __restrict__ bt_tok,
-                                                      int bt_tok_stride, const int* __restrict__ bt_pool,
-                                                      int bt_pool_stride, int nkv, int d, int dv, int ps, int num_pages,
-                                                      int num_pool_pages, int P) {
-  const int n = blockIdx.x, g = blockIdx.y, lane = threadIdx.x;
+__global__ __launch_bounds__(256) void wpa_pool_kernel(const T* __restrict__ k_pages, const T* __restrict__ v_pages,
+                                                       T* __restrict__ pk_pages, T* __restrict__ pv_pages,
+                                                       const int* __restrict__ token_seq,
+                                                       const int* __restrict__ positions, const int* __restrict__ bt_tok,
+                                                       int bt_tok_stride, const int* __restrict__ bt_pool,
+                                                       int bt_pool_stride, int nkv, int d, int dv, int ps, int num_pages,
+                                                       int num_pool_pages, int P) {
+  const int n = blockIdx.x, g = blockIdx.y;
   const int pos = positions[n];
   if ((pos + 1) % P != 0) return;
   const int s = token_seq[n];
@@ -123,20 +124,23 @@ __global__ __launch_bounds__(64) void wpa_pool_kernel(const T* __restrict__ k_pa
   T* pk = pk_pages + (((size_t)ppage * nkv + g) * E + entry) * d;
   T* pv = pv_pages + (((size_t)ppage * nkv + g) * E + entry) * dv;
   const float inv = 1.0f / (float)P;
-  const int most = d > dv ? d : dv;
-  for (int i = lane; i < most; i += 64) {
-    float ak = 0.f, av = 0.f;
+  for (int i = threadIdx.x; i < d + dv; i += 256) {
+    const bool key = i < d;
+    const int c = key ? i : i - d;
+    float acc = 0.f;
     bool bad = false;
+#pragma unroll 8
     for (int j = pos - P + 1; j <= pos; ++j) {          // in the order of the positions
       const int page = bt[j / ps];
-      if ((unsigned)page >= (unsigned)num_pages) { bad = true; break; }
-      const size_t head_page = (size_t)page * nkv + g;
-      if (i < d) ak += to_float(k_pages[(head_page * ps + (j % ps)) * d + i]);
-      if (i < dv) av += to_float(v_pages[(head_page * dv + i) * ps + (j % ps)]);
+      const bool ok = (unsigned)page < (unsigned)num_pages;
+      bad = bad || !ok;
+      const size_t head_page = (size_t)(ok ? page : 0) * nkv + g;
+      const int off = j % ps;
+      acc += key ? to_float(k_pages[(head_page * ps + off) * d + c]) : to_float(v_pages[(head_page * dv + c) * ps + off]);
     }
-    if (bad) ak = av = __uint_as_float(0x7fc00000u);     // a key of the block has no page: poison, never a stray read
-    if (i < d) pk[i] = from_float<T>(ak * inv);
-    if (i < dv) pv[i] = from_float<T>(av * inv);
+    if (bad) acc = __uint_as_float(0x7fc00000u);        // a key of the block has no page: poison, never a stray read
+    if (key) pk[c] = from_float<T>(acc * inv);
+    else pv[c] = from_float<T>(acc * inv);
   }
 }
 
@@ -152,11 +156,11 @@ extern "C" int ia_wpa_pool(const void* k_pages, const void* v_pages, void* pk_pa
     return IA_ERR_BAD_ARG;
   dim3 grid(N, nkv);
   if (dtype == IA_F32)
-    wpa_pool_kernel<float><<<grid, 64, 0, stream>>>((const float*)k_pages, (const float*)v_pages, (float*)pk_pages,
+    wpa_pool_kernel<float><<<grid, 256, 0, stream>>>((const float*)k_pages, (const float*)v_pages, (float*)pk_pages,
                                                     (float*)pv_pages, token_seq, positions, bt_tok, bt_tok_stride,
                                                     bt_pool, bt_pool_stride, nkv, d, dv, ps, num_pages, num_pool_pages, P);
   else if (dtype == IA_BF16)
-    wpa_pool_kernel<bf16_t><<<grid, 64, 0, stream>>>((const bf16_t*)k_pages, (const bf16_t*)v_pages, (bf16_t*)pk_pages,
+    wpa_pool_kernel<bf16_t><<<grid, 256, 0, stream>>>((const bf16_t*)k_pages, (const bf16_t*)v_pages, (bf16_t*)pk_pages,
                                                      (bf16_t*)pv_pages, token_seq, positions, bt_tok, bt_tok_stride,
                                                      bt_pool, bt_pool_stride, nkv, d, dv, ps, num_pages, num_pool_pages,
                                                      P);

@@ -104,43 +104,70 @@ __device__ __forceinline__ s16x4 wp_softmax_step(const f32x4& s, const bool (&ok
   return wp_s16x4(p0, p1);
 }
 
-// One tile of 16 keys, t0 .. t0 + 15, against the wave's 16 columns.  This lane's column sees the keys lo .. pos
-// (pos below zero: no such column); klo .. kmax: the keys that any column of the wave sees (the same in all lanes).
+// One tile of 16 keys, t0 .. t0 + 15, against the wave's 16 columns, in two halves so that the loads of the next tile
+// fly while this one is worked on.  klo .. kmax: the keys that any column of the wave sees (the same in all lanes).
+struct WpKeys {
+  s16x4 kr[NSK];                 // this lane's key row
+  uint2 v[NSV];                  // four keys' values of NSV channels
+  uint32_t mlo, mhi;             // which of the four are keys that some column sees
+};
+
 template <bool POW2>
-__device__ __forceinline__ void wp_tile_keys(const WpGeom& G, int t0, int j, int qd, int lo, int pos, int klo, int kmax,
-                                             float scale_log2, const s16x4 (&q)[NSK], WpCol& c, f32x4 (&o)[NSV],
+__device__ __forceinline__ void wp_load_keys(const WpGeom& G, int t0, int j, int qd, int klo, int kmax, WpKeys& T,
                                              bool& bad) {
   const int key = t0 + j;
   const int keyc = key > kmax ? kmax : (key < klo ? klo : key);
   const int page = G.bt[POW2 ? keyc >> G.ps_shift : keyc / G.ps];
   const bool page_ok = (unsigned)page < (unsigned)G.num_pages;
-  s16x4 kr[NSK];
   wp_load_row(G.k_base + (size_t)(page_ok ? page : 0) * G.k_page + (size_t)(POW2 ? keyc & (G.ps - 1) : keyc % G.ps) * WP_DIM,
-              qd, kr);
+              qd, T.kr);
   const int kg = t0 + 4 * qd;    // this lane brings the values of the keys kg .. kg + 3 (one quad, one page)
   const int kgc = kg > kmax ? (kmax & ~3) : (kg + 3 < klo ? (klo & ~3) : kg);
   const int pagev = G.bt[POW2 ? kgc >> G.ps_shift : kgc / G.ps];
   const bool pagev_ok = (unsigned)pagev < (unsigned)G.num_pages;
   const uint16_t* vq = G.v_base + (size_t)(pagev_ok ? pagev : 0) * G.v_page + (POW2 ? kgc & (G.ps - 1) : kgc % G.ps);
-  uint2 v[NSV];
 #pragma unroll
-  for (int n = 0; n < NSV; ++n) v[n] = *reinterpret_cast<const uint2*>(vq + (size_t)(n * 16 + j) * G.ps);
-  uint32_t mlo = 0u, mhi = 0u;
+  for (int n = 0; n < NSV; ++n) T.v[n] = *reinterpret_cast<const uint2*>(vq + (size_t)(n * 16 + j) * G.ps);
+  T.mlo = T.mhi = 0u;
   if (kg == kgc && pagev_ok) {
-    mlo = ((kg >= klo && kg <= kmax) ? 0x0000ffffu : 0u) | ((kg + 1 >= klo && kg + 1 <= kmax) ? 0xffff0000u : 0u);
-    mhi = ((kg + 2 >= klo && kg + 2 <= kmax) ? 0x0000ffffu : 0u) | ((kg + 3 >= klo && kg + 3 <= kmax) ? 0xffff0000u : 0u);
+    T.mlo = ((kg >= klo && kg <= kmax) ? 0x0000ffffu : 0u) | ((kg + 1 >= klo && kg + 1 <= kmax) ? 0xffff0000u : 0u);
+    T.mhi = ((kg + 2 >= klo && kg + 2 <= kmax) ? 0x0000ffffu : 0u) | ((kg + 3 >= klo && kg + 3 <= kmax) ? 0xffff0000u : 0u);
   }
   bad = bad || (key >= klo && key <= kmax && !page_ok) || (kg + 3 >= klo && kg <= kmax && !pagev_ok);
+}
+
+// This lane's column sees the keys lo .. pos (pos below zero: no such column).
+__device__ __forceinline__ void wp_use_keys(const WpKeys& T, int t0, int qd, int lo, int pos, float scale_log2,
+                                            const s16x4 (&q)[NSK], WpCol& c, f32x4 (&o)[NSV]) {
+  const int kg = t0 + 4 * qd;
   f32x4 s = (f32x4){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-  for (int st = 0; st < NSK; ++st) s = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(kr[st], q[st], s, 0, 0, 0);
+  for (int st = 0; st < NSK; ++st) s = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(T.kr[st], q[st], s, 0, 0, 0);
   bool ok[4];
 #pragma unroll
   for (int r = 0; r < 4; ++r) ok[r] = kg + r <= pos && kg + r >= lo;
   const s16x4 pw = wp_softmax_step(s, ok, scale_log2, c, o);
 #pragma unroll
   for (int n = 0; n < NSV; ++n)
-    o[n] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(wp_s16x4(v[n].x & mlo, v[n].y & mhi), pw, o[n], 0, 0, 0);
+    o[n] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(wp_s16x4(T.v[n].x & T.mlo, T.v[n].y & T.mhi), pw, o[n], 0, 0, 0);
+}
+
+// The tiles first, first + step, ... up to the one that holds key kmax, each tile's loads asked for a tile ahead.
+template <bool POW2>
+__device__ __forceinline__ void wp_walk_keys(const WpGeom& G, int first, int step, int j, int qd, int lo, int pos, int klo,
+                                             int kmax, float scale_log2, const s16x4 (&q)[NSK], WpCol& c,
+                                             f32x4 (&o)[NSV], bool& bad) {
+  if (first > kmax) return;
+  WpKeys A, B;
+  wp_load_keys<POW2>(G, first, j, qd, klo, kmax, A, bad);
+  for (int t0 = first; t0 <= kmax; t0 += 2 * step) {
+    const bool more = t0 + step <= kmax;
+    if (more) wp_load_keys<POW2>(G, t0 + step, j, qd, klo, kmax, B, bad);
+    wp_use_keys(A, t0, qd, lo, pos, scale_log2, q, c, o);
+    if (!more) break;
+    if (t0 + 2 * step <= kmax) wp_load_keys<POW2>(G, t0 + 2 * step, j, qd, klo, kmax, A, bad);
+    wp_use_keys(B, t0 + step, qd, lo, pos, scale_log2, q, c, o);
+  }
 }
 
 // One tile of 16 blocks, b0 .. b0 + 15.  This lane's column sees the blocks below nb; nbmax: the most any column sees.
@@ -260,7 +287,7 @@ __global__ __launch_bounds__(256) void wpa_prefill_kernel(
   c.l = 0.f;
   bool bad = false;
   for (int b0 = 0; b0 < nbmax; b0 += 16) wp_tile_blocks<POW2>(G, b0, j, qd, nb, nbmax, scale_log2, qr, c, o, bad);
-  for (int t0 = klo & ~15; t0 <= kmax; t0 += 16) wp_tile_keys<POW2>(G, t0, j, qd, lo, pos, klo, kmax, scale_log2, qr, c, o, bad);
+  wp_walk_keys<POW2>(G, klo & ~15, 16, j, qd, lo, pos, klo, kmax, scale_log2, qr, c, o, bad);
   float l = c.l + __shfl_xor(c.l, 16, IA_WAVE);
   l = l + __shfl_xor(l, 32, IA_WAVE);
   if (sinks) l += __builtin_amdgcn_exp2f(sinks[h] * WP_LOG2E - c.m);
@@ -306,11 +333,11 @@ __global__ __launch_bounds__(256) void wpa_decode_kernel(
   bool bad = false;
   const int lo = wp_first_key(p, window), nb = wp_blocks_seen(p, window, P);
   const int pos = col_ok ? p : -1, nbc = col_ok ? nb : 0;
-  const int block_tiles = (nb + 15) / 16, first_tile = lo / 16, key_tiles = p / 16 - first_tile + 1;
-  for (int i = wave; i < block_tiles + key_tiles; i += 4) {
-    if (i < block_tiles) wp_tile_blocks<POW2>(G, i * 16, j, qd, nbc, nb, scale_log2, qr, c, o, bad);
-    else wp_tile_keys<POW2>(G, (first_tile + i - block_tiles) * 16, j, qd, lo, pos, lo, p, scale_log2, qr, c, o, bad);
-  }
+  const int block_tiles = (nb + 15) / 16;
+  for (int i = wave; i < block_tiles; i += 4) wp_tile_blocks<POW2>(G, i * 16, j, qd, nbc, nb, scale_log2, qr, c, o, bad);
+  // the tiles of keys go round the waves from where the tiles of blocks stopped, so that no wave has two more
+  const int turn = (wave + 4 - block_tiles % 4) % 4;
+  wp_walk_keys<POW2>(G, (lo / 16 + turn) * 16, 64, j, qd, lo, pos, lo, p, scale_log2, qr, c, o, bad);
   // ---- the waves meet: a common maximum, then sums in the order of the waves
   if (qd == 0) s_m[wave][j] = c.m;
   __syncthreads();

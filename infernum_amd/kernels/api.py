@@ -1154,6 +1154,26 @@ def stream_add(h: torch.Tensor, delta) -> torch.Tensor:
     return h
 
 
+def stream_add2(h: torch.Tensor, a, b=None, x: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """h [N, H] fp32 += a, then += b (each a tensor [N, H] or a :class:`SplitSum`; b may be None), in that order, in one
+    pass; ``x`` ([N, H], either type) gets the new h."""
+    def parts_of(d):
+        return (d.parts, d.parts.shape[0]) if isinstance(d, SplitSum) else (d, 1)
+    pa, sa = parts_of(a)
+    pb, sb = parts_of(b) if b is not None else (None, 1)
+    _need(h.is_cuda and h.dtype == torch.float32 and h.is_contiguous() and pa.is_cuda and pa.is_contiguous()
+          and pa.dtype in DTYPE_CODE and pa.numel() == sa * h.numel(), "stream_add2: h fp32 [N, H], a of its shape")
+    if pb is not None:
+        _need(pb.is_cuda and pb.is_contiguous() and pb.dtype in DTYPE_CODE and pb.numel() == sb * h.numel(),
+              "stream_add2: b of h's shape")
+    if x is not None:
+        _need(x.is_cuda and x.is_contiguous() and x.dtype in DTYPE_CODE and x.shape == h.shape, "stream_add2: x like h")
+    _ok(_core().ia_stream_add2(_p(h), _p(pa), DTYPE_CODE[pa.dtype], sa, _p(pb), DTYPE_CODE[pb.dtype] if pb is not None else 0,
+                               sb, _p(x), DTYPE_CODE[x.dtype] if x is not None else 0, h.shape[0], h.shape[1], _stream()),
+        "stream_add2")
+    return h
+
+
 def add_bias(y: torch.Tensor, bias: torch.Tensor) -> torch.Tensor:
     """y [N, C] += bias [C] (fp32), in place."""
     _need(y.is_cuda and y.is_contiguous() and y.dim() == 2 and y.dtype in DTYPE_CODE, "add_bias: y [N, C]")

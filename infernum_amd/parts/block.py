@@ -201,23 +201,28 @@ class ParallelBlock(Block):
         f = None
         if self.feed_forward is not None:
             f = self.feed_forward.forward(self.feed_forward_norm.forward(h, None), ctx)
-        K.stream_add(h, a)
-        if f is not None:
-            K.stream_add(h, f)
+        # both results enter the fp32 stream in one pass, which leaves the rounded stream for the token input
         side = self.extra.get("token_input")
+        x = torch.empty(h.shape, dtype=self.rt.dtype, device=h.device) if side is not None else None
+        K.stream_add2(h, a, f, x)
         if side is not None:
-            side.forward(h, ctx)
+            side.forward(h, ctx, x=x)
         return None
 
     @staticmethod
-    def _emit_add(program, value) -> None:
+    def _emit_add(program, a, b, x) -> None:
+        """One launch per pair of forms the two results can have (a tensor, the partial sums of a split product)."""
         from ..engine.program import STREAM
         from ..kernels import api as K
         f32 = K.DTYPE_CODE[torch.float32]
-        for alt in value.alts:
-            code = f32 if alt.splits else K.DTYPE_CODE[alt.dtype]
-            program.op("core", "ia_stream_add", [program.h, alt.where, code, alt.splits or 1, program.N,
-                                                 program.hidden_size, STREAM], alt.when)
+        code = lambda alt: f32 if alt.splits else K.DTYPE_CODE[alt.dtype]       # noqa: E731
+        for aa in a.alts:
+            for bb in (b.alts if b is not None else [None]):
+                program.op("core", "ia_stream_add2",
+                           [program.h, aa.where, code(aa), aa.splits or 1, bb.where if bb is not None else None,
+                            code(bb) if bb is not None else 0, (bb.splits or 1) if bb is not None else 1, x,
+                            program.act_code if x is not None else 0, program.N, program.hidden_size, STREAM],
+                           aa.when & bb.when if bb is not None else aa.when)
 
     def native(self, program, view: CacheView) -> None:
         if type(self).forward is not ParallelBlock.forward:
@@ -232,11 +237,11 @@ class ParallelBlock(Block):
             self.feed_forward_norm.native(program, None)          # nothing pending: the norm of the same stream
             self.feed_forward.native(program, None)
             f, program.pending = program.pending, None
-        self._emit_add(program, a)
-        if f is not None:
-            self._emit_add(program, f)
-        if self.extra.get("token_input") is not None:
-            self.extra["token_input"].native(program, None)
+        side = self.extra.get("token_input")
+        x = side.stream_buffer(program) if side is not None else None
+        self._emit_add(program, a, f, x)
+        if side is not None:
+            side.native(program, None, x_ready=True)
 
 
 register_part("block", "prenorm", PreNormBlock)

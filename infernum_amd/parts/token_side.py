@@ -59,15 +59,21 @@ class GatedTableInput(Part):
         self.norm.load({n: tensors[n]})
         prepare_weights(self.rt, [(self.w_gate, None, False), (self.w_proj, None, True)])
 
-    def forward(self, h: torch.Tensor, ctx: StepContext) -> None:
-        """h [N, H] fp32, added to in place."""
-        x = K.cast(h, self.rt.dtype)
+    def forward(self, h: torch.Tensor, ctx: StepContext, x: Optional[torch.Tensor] = None) -> None:
+        """h [N, H] fp32, added to in place.  ``x``: h rounded to the compute dtype, when the caller has it already."""
+        if x is None:
+            x = K.cast(h, self.rt.dtype)
         u = linear(x, self.w_gate, kernels=self.rt.kernels)
         g = K.gelu_mul_rows(u, self.table, self.column, ctx.token_ids)
         self.norm.add_normed(h, linear(g, self.w_proj, keep_split=True, kernels=self.rt.kernels))
 
-    def native(self, program, view=None) -> None:
-        """``program.h`` is complete (nothing pending); leaves it added to."""
+    def stream_buffer(self, program):
+        """Where the program keeps the rounded stream that this part reads."""
+        return program.buffer("token_input.x", program.T * self.hidden_size * program.act_bytes)
+
+    def native(self, program, view=None, x_ready: bool = False) -> None:
+        """``program.h`` is complete (nothing pending); leaves it added to.  ``x_ready``: the rounded stream is in
+        :meth:`stream_buffer` already."""
         if type(self).forward is not GatedTableInput.forward:
             H = self.hidden_size
             program.python(lambda ctx: self.forward(program.h.view(torch.float32, ctx.num_tokens, H), ctx), type(self).__name__)
@@ -77,8 +83,9 @@ class GatedTableInput(Part):
             raise K.KernelError("token input: the stream must be complete before it is read")
         rt, N, T, H = self.rt, program.N, program.T, self.hidden_size
         program.keep(self.table)
-        x = program.buffer("token_input.x", T * H * program.act_bytes)
-        program.op("core", "ia_cast", [program.h, K.DTYPE_CODE[torch.float32], x, program.act_code, N * H, STREAM])
+        x = self.stream_buffer(program)
+        if not x_ready:
+            program.op("core", "ia_cast", [program.h, K.DTYPE_CODE[torch.float32], x, program.act_code, N * H, STREAM])
         u = emit_linear(program, x, N, self.w_gate, rt.dtype, None, False, "token_input.u", "token_input.gate").tensor()
         program.op("core", "ia_gelu_mul_rows", [u, u, program.act_code, self.table, K.DTYPE_CODE[self.table.dtype],
                                                 self.columns, self.column, program.token_ids, self.vocab_size, N,
