@@ -26,6 +26,7 @@
 #include "common.h"
 
 #define WPA_MAX_D 640
+#define WPA_POOL_CHUNK 512      // positions of a block whose places are looked up together
 
 template <typename T>
 __global__ __launch_bounds__(64) void wpa_prepare_kernel(
@@ -103,7 +104,7 @@ extern "C" int ia_wpa_prepare(const void* src, int src_stride, const float* bias
 }
 
 // grid (N, nkv), 256 threads: a thread a value of the block's key or value, the block's positions added in their
-// order (the loads of several are in flight together).  A token that is not the last of its block leaves at once.
+// order (the loads of sixteen are in flight together).  A token that is not the last of its block leaves at once.
 template <typename T>
 __global__ __launch_bounds__(256) void wpa_pool_kernel(const T* __restrict__ k_pages, const T* __restrict__ v_pages,
                                                        T* __restrict__ pk_pages, T* __restrict__ pv_pages,
@@ -111,8 +112,12 @@ __global__ __launch_bounds__(256) void wpa_pool_kernel(const T* __restrict__ k_p
                                                        const int* __restrict__ positions, const int* __restrict__ bt_tok,
                                                        int bt_tok_stride, const int* __restrict__ bt_pool,
                                                        int bt_pool_stride, int nkv, int d, int dv, int ps, int num_pages,
-                                                       int num_pool_pages, int P) {
-  const int n = blockIdx.x, g = blockIdx.y;
+                                                       int num_pool_pages, int P, int N, int stride) {
+  // The tokens that close a block stand P apart; workgroups go to dies and compute units by their number in turn,
+  // so with tokens in the order of the workgroups a block size that shares factors with those turns would send all
+  // the work to a few compute units (blocks of 64 in a prompt of 2,048: four of 256).  The tokens are dealt out in
+  // steps of a number that shares no factor with N instead.
+  const int n = (int)(((long long)blockIdx.x * stride) % N), g = blockIdx.y;
   const int pos = positions[n];
   if ((pos + 1) % P != 0) return;
   const int s = token_seq[n];
@@ -124,23 +129,56 @@ __global__ __launch_bounds__(256) void wpa_pool_kernel(const T* __restrict__ k_p
   T* pk = pk_pages + (((size_t)ppage * nkv + g) * E + entry) * d;
   T* pv = pv_pages + (((size_t)ppage * nkv + g) * E + entry) * dv;
   const float inv = 1.0f / (float)P;
-  for (int i = threadIdx.x; i < d + dv; i += 256) {
-    const bool key = i < d;
-    const int c = key ? i : i - d;
-    float acc = 0.f;
-    bool bad = false;
-#pragma unroll 8
-    for (int j = pos - P + 1; j <= pos; ++j) {          // in the order of the positions
-      const int page = bt[j / ps];
+  // where each of the block's positions lies, found once for all values: the sums' loads then wait for nothing
+  __shared__ int s_page[WPA_POOL_CHUNK], s_off[WPA_POOL_CHUNK];
+  __shared__ int s_bad;
+  if (threadIdx.x == 0) s_bad = 0;
+  float acc[(WPA_MAX_D * 2 + 255) / 256];
+#pragma unroll
+  for (int u = 0; u < (WPA_MAX_D * 2 + 255) / 256; ++u) acc[u] = 0.f;
+  for (int j0 = pos - P + 1; j0 <= pos; j0 += WPA_POOL_CHUNK) {
+    const int cnt = pos - j0 + 1 < WPA_POOL_CHUNK ? pos - j0 + 1 : WPA_POOL_CHUNK;
+    __syncthreads();
+    for (int t = threadIdx.x; t < cnt; t += 256) {
+      const int j = j0 + t, page = bt[j / ps];
       const bool ok = (unsigned)page < (unsigned)num_pages;
-      bad = bad || !ok;
-      const size_t head_page = (size_t)(ok ? page : 0) * nkv + g;
-      const int off = j % ps;
-      acc += key ? to_float(k_pages[(head_page * ps + off) * d + c]) : to_float(v_pages[(head_page * dv + c) * ps + off]);
+      if (!ok) s_bad = 1;
+      s_page[t] = ok ? page : 0;
+      s_off[t] = j % ps;
     }
-    if (bad) acc = __uint_as_float(0x7fc00000u);        // a key of the block has no page: poison, never a stray read
-    if (key) pk[c] = from_float<T>(acc * inv);
-    else pv[c] = from_float<T>(acc * inv);
+    __syncthreads();
+#pragma unroll
+    for (int u = 0; u < (WPA_MAX_D * 2 + 255) / 256; ++u) {
+      const int i = threadIdx.x + 256 * u;
+      if (i >= d + dv) break;
+      const bool key = i < d;
+      const int c = key ? i : i - d;
+      float a = acc[u];
+      for (int t = 0; t < cnt; t += 16) {                 // sixteen loads are out before the first is added
+        float x[16];
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          const int tt = t + e < cnt ? t + e : cnt - 1;
+          const size_t head_page = (size_t)s_page[tt] * nkv + g;
+          // one load from a chosen address, not a choice between two loads: nothing waits between the sixteen
+          const T* at = key ? k_pages + (head_page * ps + s_off[tt]) * d + c : v_pages + (head_page * dv + c) * ps + s_off[tt];
+          x[e] = to_float(*at);
+        }
+#pragma unroll
+        for (int e = 0; e < 16; ++e) a += t + e < cnt ? x[e] : 0.f;      // in the order of the positions
+      }
+      acc[u] = a;
+    }
+  }
+  __syncthreads();
+  const bool bad = s_bad != 0;                             // a key of the block has no page: poison, never a stray read
+#pragma unroll
+  for (int u = 0; u < (WPA_MAX_D * 2 + 255) / 256; ++u) {
+    const int i = threadIdx.x + 256 * u;
+    if (i >= d + dv) break;
+    const float r = bad ? __uint_as_float(0x7fc00000u) : acc[u] * inv;
+    if (i < d) pk[i] = from_float<T>(r);
+    else pv[i - d] = from_float<T>(r);
   }
 }
 
@@ -155,15 +193,19 @@ extern "C" int ia_wpa_pool(const void* k_pages, const void* v_pages, void* pk_pa
   if (!k_pages || !v_pages || !pk_pages || !pv_pages || !token_seq || !positions || !bt_tok || !bt_pool)
     return IA_ERR_BAD_ARG;
   dim3 grid(N, nkv);
+  int stride = 1;
+  for (int prime : {7919, 104729, 1299709})
+    if (N % prime != 0) { stride = prime; break; }
   if (dtype == IA_F32)
     wpa_pool_kernel<float><<<grid, 256, 0, stream>>>((const float*)k_pages, (const float*)v_pages, (float*)pk_pages,
                                                     (float*)pv_pages, token_seq, positions, bt_tok, bt_tok_stride,
-                                                    bt_pool, bt_pool_stride, nkv, d, dv, ps, num_pages, num_pool_pages, P);
+                                                    bt_pool, bt_pool_stride, nkv, d, dv, ps, num_pages, num_pool_pages, P,
+                                                    N, stride);
   else if (dtype == IA_BF16)
     wpa_pool_kernel<bf16_t><<<grid, 256, 0, stream>>>((const bf16_t*)k_pages, (const bf16_t*)v_pages, (bf16_t*)pk_pages,
                                                      (bf16_t*)pv_pages, token_seq, positions, bt_tok, bt_tok_stride,
                                                      bt_pool, bt_pool_stride, nkv, d, dv, ps, num_pages, num_pool_pages,
-                                                     P);
+                                                     P, N, stride);
   else
     return IA_ERR_BAD_ARG;
   IA_LAUNCH_CHECK();

@@ -17,9 +17,9 @@
 // block b lies in the page of its last position t = b P + P - 1 at place (t % page_size) / P; neighbouring blocks need
 // not be neighbours there, so a block's values are fetched one by one (there are few blocks: a position in P).
 //
-// Portions of prompts: a wave takes 16 consecutive rows of one query head, a workgroup a tile of 64 rows.  Single
-// tokens: the 16 columns are up to 16 query heads of one key/value head of one token; the tiles (of blocks, then of
-// keys) are dealt out over the four waves of a workgroup, which join through LDS in the order of the waves.
+// The 16 columns are 16 consecutive rows of one query head (portions of prompts) or up to 16 query heads of one
+// key/value head of one token (single tokens); the tiles (of blocks, then of keys) are dealt out over the four waves
+// of a workgroup, which join through LDS in the order of the waves.
 // Values of keys that no column of the tile sees are zeroed after the load and their weights are zero: a page that
 // went back to the pool never leaks in.  A key that is needed but has no page in the block table gives NaN.
 #include "common.h"
@@ -153,20 +153,23 @@ __device__ __forceinline__ void wp_use_keys(const WpKeys& T, int t0, int qd, int
 }
 
 // The tiles first, first + step, ... up to the one that holds key kmax, each tile's loads asked for a tile ahead.
-template <bool POW2>
+// CT: query heads of one key/value head that the wave takes for its rows; a tile that was loaded serves them all.
+template <bool POW2, int CT>
 __device__ __forceinline__ void wp_walk_keys(const WpGeom& G, int first, int step, int j, int qd, int lo, int pos, int klo,
-                                             int kmax, float scale_log2, const s16x4 (&q)[NSK], WpCol& c,
-                                             f32x4 (&o)[NSV], bool& bad) {
+                                             int kmax, float scale_log2, const s16x4 (&q)[CT][NSK], WpCol (&c)[CT],
+                                             f32x4 (&o)[CT][NSV], bool& bad) {
   if (first > kmax) return;
   WpKeys A, B;
   wp_load_keys<POW2>(G, first, j, qd, klo, kmax, A, bad);
   for (int t0 = first; t0 <= kmax; t0 += 2 * step) {
     const bool more = t0 + step <= kmax;
     if (more) wp_load_keys<POW2>(G, t0 + step, j, qd, klo, kmax, B, bad);
-    wp_use_keys(A, t0, qd, lo, pos, scale_log2, q, c, o);
+#pragma unroll
+    for (int u = 0; u < CT; ++u) wp_use_keys(A, t0, qd, lo, pos, scale_log2, q[u], c[u], o[u]);
     if (!more) break;
     if (t0 + 2 * step <= kmax) wp_load_keys<POW2>(G, t0 + 2 * step, j, qd, klo, kmax, A, bad);
-    wp_use_keys(B, t0 + step, qd, lo, pos, scale_log2, q, c, o);
+#pragma unroll
+    for (int u = 0; u < CT; ++u) wp_use_keys(B, t0 + step, qd, lo, pos, scale_log2, q[u], c[u], o[u]);
   }
 }
 
@@ -249,8 +252,12 @@ __device__ __forceinline__ void wp_store_bf16x4(uint16_t* at, const f32x4& x, fl
 }
 
 // ------------------------------------------------------------------------ portions of prompts
-// 256 threads; a workgroup is one tile (request, first row) of 64 rows and one query head; wave w takes the rows
-// first + 16 w .. + 15.  Workgroups are numbered so that the heads of one tile follow each other.
+// 256 threads; a workgroup takes 16 consecutive rows of one query head (a quarter of a tile (request, first row) of 64
+// rows that the host lists): the 16 columns are those rows, and the tiles of blocks and of keys are dealt out over the
+// four waves, which join through LDS in the order of the waves, as for single tokens.  A wave alone on 16 rows would
+// walk up to window / 16 tiles one after the other, each a chain of dependent matrix instructions, exchanges and
+// exponentials, with two such waves a SIMD at 2,048 rows and 16 heads: the rows' keys in four parts make four times
+// the waves, which hide each other's waits.  Workgroups are numbered so that the heads of one tile follow each other.
 template <bool POW2>
 __global__ __launch_bounds__(256) void wpa_prefill_kernel(
     const uint16_t* __restrict__ q, int q_stride, const uint16_t* __restrict__ k_pages,
@@ -259,13 +266,18 @@ __global__ __launch_bounds__(256) void wpa_prefill_kernel(
     const int* __restrict__ seq_ctx, const int* __restrict__ bt_tok, int bt_tok_stride, const int* __restrict__ bt_pool,
     int bt_pool_stride, const int* __restrict__ tiles, int nh, int nkv, int ps, int num_pages, int num_pool_pages,
     float scale_log2, int window, int P) {
+  __shared__ f32x4 red[3][NSV][64];
+  __shared__ float s_m[4][16], s_l[4][64];
+  __shared__ int s_bad;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, j = lane & 15, qd = lane >> 4;
   const int lin = blockIdx.x;
-  const int tile = lin / nh, h = lin - tile * nh;
+  const int tile = lin / (4 * nh), rest = lin - tile * 4 * nh;
+  const int sub = rest / nh, h = rest - sub * nh;
   const int sidx = tiles[2 * tile], row0 = tiles[2 * tile + 1];
   const int qstart = seq_starts[sidx], qlen = seq_starts[sidx + 1] - qstart, ctx = seq_ctx[sidx];
-  const int rb = row0 + wave * 16;
-  if (rb >= qlen) return;                                   // the waves share nothing: no barrier follows
+  const int rb = row0 + sub * 16;
+  if (rb >= qlen) return;                                   // the whole workgroup: no barrier has been met
+  if (tid == 0) s_bad = 0;
   const int g = h / (nh / nkv);
   const int row = rb + j;
   const bool col_ok = row < qlen;
@@ -277,23 +289,47 @@ __global__ __launch_bounds__(256) void wpa_prefill_kernel(
   const WpGeom G = wp_geom(k_pages, v_pages, pk_pages, pv_pages, bt_tok, bt_tok_stride, bt_pool, bt_pool_stride, sidx, g,
                            nkv, ps, num_pages, num_pool_pages, P);
   const size_t qrow = (size_t)(qstart + (col_ok ? row : rb));
-  s16x4 qr[NSK];
+  s16x4 qr1[1][NSK];
+  s16x4 (&qr)[NSK] = qr1[0];
   wp_load_row(q + qrow * q_stride + (size_t)h * WP_DIM, qd, qr);
-  f32x4 o[NSV];
+  f32x4 o1[1][NSV];
+  f32x4 (&o)[NSV] = o1[0];
 #pragma unroll
   for (int n = 0; n < NSV; ++n) o[n] = (f32x4){0.f, 0.f, 0.f, 0.f};
-  WpCol c;
+  WpCol c1[1];
+  WpCol& c = c1[0];
   c.m = -INFINITY;
   c.l = 0.f;
   bool bad = false;
-  for (int b0 = 0; b0 < nbmax; b0 += 16) wp_tile_blocks<POW2>(G, b0, j, qd, nb, nbmax, scale_log2, qr, c, o, bad);
-  wp_walk_keys<POW2>(G, klo & ~15, 16, j, qd, lo, pos, klo, kmax, scale_log2, qr, c, o, bad);
-  float l = c.l + __shfl_xor(c.l, 16, IA_WAVE);
-  l = l + __shfl_xor(l, 32, IA_WAVE);
-  if (sinks) l += __builtin_amdgcn_exp2f(sinks[h] * WP_LOG2E - c.m);
+  const int block_tiles = (nbmax + 15) / 16;
+  for (int i = wave; i < block_tiles; i += 4) wp_tile_blocks<POW2>(G, i * 16, j, qd, nb, nbmax, scale_log2, qr, c, o, bad);
+  const int turn = (wave + 4 - block_tiles % 4) % 4;
+  wp_walk_keys<POW2, 1>(G, (klo / 16 + turn) * 16, 64, j, qd, lo, pos, klo, kmax, scale_log2, qr1, c1, o1, bad);
+  // ---- the waves meet: a common maximum, then sums in the order of the waves
+  if (qd == 0) s_m[wave][j] = c.m;
+  __syncthreads();
+  if (bad) s_bad = 1;
+  const float M = fmaxf(fmaxf(s_m[0][j], s_m[1][j]), fmaxf(s_m[2][j], s_m[3][j]));
+  const float f = (c.m == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(c.m - M);
+#pragma unroll
+  for (int n = 0; n < NSV; ++n) o[n] *= f;
+  s_l[wave][lane] = c.l * f;
+  if (wave > 0) {
+#pragma unroll
+    for (int n = 0; n < NSV; ++n) red[wave - 1][n][lane] = o[n];
+  }
+  __syncthreads();
+  if (wave > 0 || !col_ok) return;
+#pragma unroll
+  for (int n = 0; n < NSV; ++n) o[n] = ((o[n] + red[0][n][lane]) + red[1][n][lane]) + red[2][n][lane];
+  float l = 0.f;
+#pragma unroll
+  for (int w = 0; w < 4; ++w)
+#pragma unroll
+    for (int x = 0; x < 4; ++x) l += s_l[w][x * 16 + j];
+  if (sinks) l += __builtin_amdgcn_exp2f(sinks[h] * WP_LOG2E - M);
   float inv = 1.0f / l;
-  if (__any(bad)) inv = __uint_as_float(0x7fc00000u);
-  if (!col_ok) return;
+  if (s_bad) inv = __uint_as_float(0x7fc00000u);
   uint16_t* at = out + (qrow * nh + h) * WP_VDIM + 4 * qd;
 #pragma unroll
   for (int n = 0; n < NSV; ++n) wp_store_bf16x4(at + n * 16, o[n], inv);
@@ -322,12 +358,15 @@ __global__ __launch_bounds__(256) void wpa_decode_kernel(
   if (tid == 0) s_bad = 0;
   const WpGeom G = wp_geom(k_pages, v_pages, pk_pages, pv_pages, bt_tok, bt_tok_stride, bt_pool, bt_pool_stride, b, g, nkv,
                            ps, num_pages, num_pool_pages, P);
-  s16x4 qr[NSK];
+  s16x4 qr1[1][NSK];
+  s16x4 (&qr)[NSK] = qr1[0];
   wp_load_row(q + (size_t)b * q_stride + (size_t)h * WP_DIM, qd, qr);
-  f32x4 o[NSV];
+  f32x4 o1[1][NSV];
+  f32x4 (&o)[NSV] = o1[0];
 #pragma unroll
   for (int n = 0; n < NSV; ++n) o[n] = (f32x4){0.f, 0.f, 0.f, 0.f};
-  WpCol c;
+  WpCol c1[1];
+  WpCol& c = c1[0];
   c.m = -INFINITY;
   c.l = 0.f;
   bool bad = false;
@@ -337,7 +376,7 @@ __global__ __launch_bounds__(256) void wpa_decode_kernel(
   for (int i = wave; i < block_tiles; i += 4) wp_tile_blocks<POW2>(G, i * 16, j, qd, nbc, nb, scale_log2, qr, c, o, bad);
   // the tiles of keys go round the waves from where the tiles of blocks stopped, so that no wave has two more
   const int turn = (wave + 4 - block_tiles % 4) % 4;
-  wp_walk_keys<POW2>(G, (lo / 16 + turn) * 16, 64, j, qd, lo, pos, lo, p, scale_log2, qr, c, o, bad);
+  wp_walk_keys<POW2, 1>(G, (lo / 16 + turn) * 16, 64, j, qd, lo, pos, lo, p, scale_log2, qr1, c1, o1, bad);
   // ---- the waves meet: a common maximum, then sums in the order of the waves
   if (qd == 0) s_m[wave][j] = c.m;
   __syncthreads();
@@ -398,8 +437,9 @@ extern "C" int ia_wpa_prefill(const void* q, int q_stride, const void* k_pages, 
   if (!q || !k_pages || !v_pages || !out || !tiles || !seq_starts || !seq_ctx || !bt_tok) return IA_ERR_BAD_ARG;
   if ((long long)num_tiles * nh > 0x7fffffffLL) return IA_ERR_UNSUPPORTED;
   if (!(window > 0 && P > 0)) P = 0;
+  if ((long long)num_tiles * nh * 4 > 0x7fffffffLL) return IA_ERR_UNSUPPORTED;
 #define WP_PRE(P2)                                                                                                 \
-  wpa_prefill_kernel<P2><<<num_tiles * nh, 256, 0, stream>>>(                                                      \
+  wpa_prefill_kernel<P2><<<num_tiles * nh * 4, 256, 0, stream>>>(                                                  \
       (const uint16_t*)q, q_stride, (const uint16_t*)k_pages, (const uint16_t*)v_pages, (const uint16_t*)pk_pages, \
       (const uint16_t*)pv_pages, (uint16_t*)out, sinks, seq_starts, seq_ctx, bt_tok, bt_tok_stride, bt_pool,       \
       bt_pool_stride, tiles, nh, nkv, ps, num_pages, num_pool_pages, scale * WP_LOG2E, window, P)
