@@ -173,7 +173,9 @@ def library_plan(name: str) -> Dict:
         if not (d.isdigit() and v.isdigit() and int(d) in SUPPORTED_HEAD_DIMS and int(v) in SUPPORTED_HEAD_DIMS):
             raise BuildError(f"no MFMA window-and-blocks attention kernel named {name!r}: key and value sizes are "
                              "multiples of 16 up to 256")
-        return {"sources": ["window_pool_attention_mfma.hip"], "defines": [f"-DWP_DIM={int(d)}", f"-DWP_VDIM={int(v)}"]}
+        # accumulators in ordinary vector registers, as for attn_d<D>: the running softmax rescales them
+        return {"sources": ["window_pool_attention_mfma.hip"],
+                "defines": [f"-DWP_DIM={int(d)}", f"-DWP_VDIM={int(v)}", "-mllvm", "-amdgpu-mfma-vgpr-form"]}
     raise BuildError(f"unknown library {name!r}")
 
 

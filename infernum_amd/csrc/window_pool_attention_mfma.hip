@@ -97,9 +97,13 @@ __device__ __forceinline__ s16x4 wp_softmax_step(const f32x4& s, const bool (&ok
   const uint32_t p1 = __builtin_bit_cast(uint32_t, __builtin_convertvector(w1, bf16x2_t));
   const float sum = (bf16_bits_to_float((uint16_t)(p0 & 0xffffu)) + bf16_bits_to_float((uint16_t)(p0 >> 16))) +
                     (bf16_bits_to_float((uint16_t)(p1 & 0xffffu)) + bf16_bits_to_float((uint16_t)(p1 >> 16)));
-  c.l = c.l * corr + sum;
+  // most tiles leave every column's maximum where it was: the accumulators are rescaled only when one has moved
+  if (__any(m_new != c.m)) {
+    c.l *= corr;
 #pragma unroll
-  for (int n = 0; n < NSV; ++n) o[n] *= corr;
+    for (int n = 0; n < NSV; ++n) o[n] *= corr;
+  }
+  c.l += sum;
   c.m = m_new;
   return wp_s16x4(p0, p1);
 }
@@ -154,11 +158,21 @@ __device__ __forceinline__ void wp_use_keys(const WpKeys& T, int t0, int qd, int
 
 // The tiles first, first + step, ... up to the one that holds key kmax, each tile's loads asked for a tile ahead.
 // CT: query heads of one key/value head that the wave takes for its rows; a tile that was loaded serves them all.
-template <bool POW2, int CT>
+// AHEAD false: no tile is asked for ahead.
+template <bool POW2, int CT, bool AHEAD>
 __device__ __forceinline__ void wp_walk_keys(const WpGeom& G, int first, int step, int j, int qd, int lo, int pos, int klo,
                                              int kmax, float scale_log2, const s16x4 (&q)[CT][NSK], WpCol (&c)[CT],
                                              f32x4 (&o)[CT][NSV], bool& bad) {
   if (first > kmax) return;
+  if (!AHEAD) {                  // a tile's loads and its work in turn: fewer registers, so more waves share a SIMD
+    for (int t0 = first; t0 <= kmax; t0 += step) {
+      WpKeys A;
+      wp_load_keys<POW2>(G, t0, j, qd, klo, kmax, A, bad);
+#pragma unroll
+      for (int u = 0; u < CT; ++u) wp_use_keys(A, t0, qd, lo, pos, scale_log2, q[u], c[u], o[u]);
+    }
+    return;
+  }
   WpKeys A, B;
   wp_load_keys<POW2>(G, first, j, qd, klo, kmax, A, bad);
   for (int t0 = first; t0 <= kmax; t0 += 2 * step) {
@@ -186,8 +200,17 @@ __device__ __forceinline__ void wp_tile_blocks(const WpGeom& G, int b0, int j, i
   wp_load_row(G.pk_base + (size_t)(page_ok ? page : 0) * G.pk_page + (size_t)((POW2 ? t & (G.ps - 1) : t % G.ps) / G.P) * WP_DIM,
               qd, kr);
   bad = bad || (b0 + j < nbmax && !page_ok);
-  // the values of the blocks b0 + 4 qd .. + 3, channel by channel
-  uint16_t vv[NSV][4];
+  f32x4 s = (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int st = 0; st < NSK; ++st) s = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(kr[st], q[st], s, 0, 0, 0);
+  bool ok[4];
+#pragma unroll
+  for (int r = 0; r < 4; ++r) ok[r] = b0 + 4 * qd + r < nb;
+  const s16x4 pw = wp_softmax_step(s, ok, scale_log2, c, o);
+  // the values of the blocks b0 + 4 qd .. + 3, channel by channel, fetched after the scores are done with their
+  // registers (blocks are few; what counts is that this path needs no more registers than the keys')
+  const uint16_t* vr[4];
+  bool have[4];
 #pragma unroll
   for (int r = 0; r < 4; ++r) {
     const int bb = b0 + 4 * qd + r;
@@ -196,23 +219,16 @@ __device__ __forceinline__ void wp_tile_blocks(const WpGeom& G, int b0, int j, i
     const int pg = G.btp[POW2 ? tt >> G.ps_shift : tt / G.ps];
     const bool pg_ok = (unsigned)pg < (unsigned)G.num_pool_pages;
     bad = bad || (in && !pg_ok);
-    const uint16_t* vr = G.pv_base + (size_t)(pg_ok ? pg : 0) * G.pv_page +
-                         (size_t)((POW2 ? tt & (G.ps - 1) : tt % G.ps) / G.P) * WP_VDIM + j;
-#pragma unroll
-    for (int n = 0; n < NSV; ++n) vv[n][r] = (in && pg_ok) ? vr[n * 16] : (uint16_t)0;
+    have[r] = in && pg_ok;
+    vr[r] = G.pv_base + (size_t)(pg_ok ? pg : 0) * G.pv_page + (size_t)((POW2 ? tt & (G.ps - 1) : tt % G.ps) / G.P) * WP_VDIM + j;
   }
-  f32x4 s = (f32x4){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-  for (int st = 0; st < NSK; ++st) s = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(kr[st], q[st], s, 0, 0, 0);
-  bool ok[4];
+  for (int n = 0; n < NSV; ++n) {
+    uint32_t x[4];
 #pragma unroll
-  for (int r = 0; r < 4; ++r) ok[r] = b0 + 4 * qd + r < nb;
-  const s16x4 pw = wp_softmax_step(s, ok, scale_log2, c, o);
-#pragma unroll
-  for (int n = 0; n < NSV; ++n)
-    o[n] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(
-        wp_s16x4((uint32_t)vv[n][0] | ((uint32_t)vv[n][1] << 16), (uint32_t)vv[n][2] | ((uint32_t)vv[n][3] << 16)), pw,
-        o[n], 0, 0, 0);
+    for (int r = 0; r < 4; ++r) x[r] = have[r] ? (uint32_t)vr[r][n * 16] : 0u;
+    o[n] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(wp_s16x4(x[0] | (x[1] << 16), x[2] | (x[3] << 16)), pw, o[n], 0, 0, 0);
+  }
 }
 
 __device__ __forceinline__ WpGeom wp_geom(const uint16_t* k_pages, const uint16_t* v_pages, const uint16_t* pk_pages,
@@ -257,7 +273,9 @@ __device__ __forceinline__ void wp_store_bf16x4(uint16_t* at, const f32x4& x, fl
 // four waves, which join through LDS in the order of the waves, as for single tokens.  A wave alone on 16 rows would
 // walk up to window / 16 tiles one after the other, each a chain of dependent matrix instructions, exchanges and
 // exponentials, with two such waves a SIMD at 2,048 rows and 16 heads: the rows' keys in four parts make four times
-// the waves, which hide each other's waits.  Workgroups are numbered so that the heads of one tile follow each other.
+// the waves, and without a tile asked for ahead the kernel's registers let three of them share a SIMD (at head sizes
+// of 128: 139 registers; held to the 128 of four waves, a dozen values went to scratch and nothing was gained).
+// Workgroups are numbered so that the heads of one tile follow each other.
 template <bool POW2>
 __global__ __launch_bounds__(256) void wpa_prefill_kernel(
     const uint16_t* __restrict__ q, int q_stride, const uint16_t* __restrict__ k_pages,
@@ -304,7 +322,7 @@ __global__ __launch_bounds__(256) void wpa_prefill_kernel(
   const int block_tiles = (nbmax + 15) / 16;
   for (int i = wave; i < block_tiles; i += 4) wp_tile_blocks<POW2>(G, i * 16, j, qd, nb, nbmax, scale_log2, qr, c, o, bad);
   const int turn = (wave + 4 - block_tiles % 4) % 4;
-  wp_walk_keys<POW2, 1>(G, (klo / 16 + turn) * 16, 64, j, qd, lo, pos, klo, kmax, scale_log2, qr1, c1, o1, bad);
+  wp_walk_keys<POW2, 1, false>(G, (klo / 16 + turn) * 16, 64, j, qd, lo, pos, klo, kmax, scale_log2, qr1, c1, o1, bad);
   // ---- the waves meet: a common maximum, then sums in the order of the waves
   if (qd == 0) s_m[wave][j] = c.m;
   __syncthreads();
@@ -376,7 +394,7 @@ __global__ __launch_bounds__(256) void wpa_decode_kernel(
   for (int i = wave; i < block_tiles; i += 4) wp_tile_blocks<POW2>(G, i * 16, j, qd, nbc, nb, scale_log2, qr, c, o, bad);
   // the tiles of keys go round the waves from where the tiles of blocks stopped, so that no wave has two more
   const int turn = (wave + 4 - block_tiles % 4) % 4;
-  wp_walk_keys<POW2, 1>(G, (lo / 16 + turn) * 16, 64, j, qd, lo, pos, lo, p, scale_log2, qr1, c1, o1, bad);
+  wp_walk_keys<POW2, 1, true>(G, (lo / 16 + turn) * 16, 64, j, qd, lo, pos, lo, p, scale_log2, qr1, c1, o1, bad);
   // ---- the waves meet: a common maximum, then sums in the order of the waves
   if (qd == 0) s_m[wave][j] = c.m;
   __syncthreads();
