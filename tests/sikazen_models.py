@@ -72,8 +72,8 @@ S4 = {"architecture": "Sikazen", "vocab": 150, "width": 80, "norm": {"eps": 1e-6
       "layers": [_layer("hgrn2", _hgrn2(5, 16, 16), 64), _layer("hgrn2", _hgrn2(2, 40, 48), 48)]}
 S5 = {"architecture": "Sikazen", "vocab": 1100, "width": 48, "embedding": {"scale": 2.0}, "norm": {"eps": 1e-5},
       "layers": [_layer("attention", _attn(3, 3, 48, 16, 0.15, _rot(10000.0, 48)), 64),
-                 _layer("attention", _attn(4, 2, 16, 16, 0.25, _rot(10000.0, 16, 4.0), 33, 16)),
-                 _layer("latent_attention", _latent(1, 48, 16, 64, 96, 32, 0.1, 250000.0), 32)]}
+                 _layer("attention", _attn(4, 2, 16, 16, 0.25, _rot(10000.0, 16, 3.0), 33, 16)),
+                 _layer("latent_attention", _latent(1, 48, 16, 64, 80, 32, 0.1, 300000.0), 32)]}
 RAW = {"S1": S1, "S2": S2, "S3": S3, "S4": S4, "S5": S5}
 SEED = {"S1": 5, "S2": 6, "S3": 7, "S4": 15, "S5": 9}
 

@@ -311,7 +311,7 @@ def test_sinks_in_the_matrix_core_kernels_against_the_plain_kernel(nh, nkv, d, p
     assert rel_err(got, want.double().cpu()) <= 3e-2
 
 
-@pytest.mark.parametrize("nh,nkv,d,dv,ps,window,pool", [(4, 2, 16, 32, 4, 20, 6), (6, 2, 64, 64, 16, 72, 12), (20, 1, 32, 16, 8, 1, 1),
+@pytest.mark.parametrize("nh,nkv,d,dv,ps,window,pool", [(4, 2, 16, 32, 4, 20, 6), (6, 2, 64, 64, 16, 40, 10), (20, 1, 32, 16, 8, 1, 1),
                                                         (3, 3, 48, 16, 12, 0, 0), (4, 2, 16, 16, 16, 33, 16), (2, 1, 128, 128, 16, 7, 9),
                                                         (17, 1, 16, 16, 4, 40, 5)])
 def test_window_and_blocks_on_the_matrix_cores_against_the_plain_kernel(nh, nkv, d, dv, ps, window, pool):
