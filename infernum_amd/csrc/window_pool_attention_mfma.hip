@@ -156,20 +156,99 @@ __device__ __forceinline__ void wp_use_keys(const WpKeys& T, int t0, int qd, int
     o[n] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(wp_s16x4(T.v[n].x & T.mlo, T.v[n].y & T.mhi), pw, o[n], 0, 0, 0);
 }
 
+// A tile without look ahead, in the halves of its loads: the keys, then (wp_work_tile) the values, both asked for before
+// the first product.  Asking for the next tile's keys a tile ahead was measured too: 17 registers more, still three
+// waves a SIMD, and 8% slower.  ``inner``: every column of the wave sees the tile whole and it lies in one page (pages of a multiple of 16 positions): the page is looked up
+// once for the wave, the addresses are the wave's plus a lane's place, and neither scores, weights nor values need a
+// mask.  Most tiles of a window are such tiles.
+template <bool POW2>
+__device__ __forceinline__ void wp_load_k(const WpGeom& G, int t0, int j, int qd, int klo, int kmax, bool inner,
+                                          s16x4 (&kr)[NSK], bool& bad) {
+  if (inner) {
+    const int page = G.bt[POW2 ? t0 >> G.ps_shift : t0 / G.ps];
+    const bool page_ok = (unsigned)page < (unsigned)G.num_pages;
+    bad = bad || !page_ok;
+    const int off = POW2 ? t0 & (G.ps - 1) : t0 % G.ps;
+    wp_load_row(G.k_base + (size_t)(page_ok ? page : 0) * G.k_page + (size_t)off * WP_DIM + j * WP_DIM, qd, kr);
+    return;
+  }
+  const int key = t0 + j;
+  const int keyc = key > kmax ? kmax : (key < klo ? klo : key);
+  const int page = G.bt[POW2 ? keyc >> G.ps_shift : keyc / G.ps];
+  const bool page_ok = (unsigned)page < (unsigned)G.num_pages;
+  wp_load_row(G.k_base + (size_t)(page_ok ? page : 0) * G.k_page + (size_t)(POW2 ? keyc & (G.ps - 1) : keyc % G.ps) * WP_DIM,
+              qd, kr);
+  bad = bad || (key >= klo && key <= kmax && !page_ok);
+}
+
+template <bool POW2>
+__device__ __forceinline__ void wp_load_v(const WpGeom& G, int t0, int j, int qd, int klo, int kmax, bool inner,
+                                          uint2 (&v)[NSV], uint32_t& mlo, uint32_t& mhi, bool& bad) {
+  if (inner) {
+    const int page = G.bt[POW2 ? t0 >> G.ps_shift : t0 / G.ps];
+    const bool page_ok = (unsigned)page < (unsigned)G.num_pages;
+    bad = bad || !page_ok;
+    const int off = POW2 ? t0 & (G.ps - 1) : t0 % G.ps;
+    const uint16_t* vq = G.v_base + (size_t)(page_ok ? page : 0) * G.v_page + off + (size_t)j * G.ps + 4 * qd;
+#pragma unroll
+    for (int n = 0; n < NSV; ++n) v[n] = *reinterpret_cast<const uint2*>(vq + (size_t)n * 16 * G.ps);
+    mlo = mhi = 0xffffffffu;
+    return;
+  }
+  const int kg = t0 + 4 * qd;    // this lane brings the values of the keys kg .. kg + 3 (one quad, one page)
+  const int kgc = kg > kmax ? (kmax & ~3) : (kg + 3 < klo ? (klo & ~3) : kg);
+  const int pagev = G.bt[POW2 ? kgc >> G.ps_shift : kgc / G.ps];
+  const bool pagev_ok = (unsigned)pagev < (unsigned)G.num_pages;
+  const uint16_t* vq = G.v_base + (size_t)(pagev_ok ? pagev : 0) * G.v_page + (POW2 ? kgc & (G.ps - 1) : kgc % G.ps);
+#pragma unroll
+  for (int n = 0; n < NSV; ++n) v[n] = *reinterpret_cast<const uint2*>(vq + (size_t)(n * 16 + j) * G.ps);
+  mlo = mhi = 0u;
+  if (kg == kgc && pagev_ok) {
+    mlo = ((kg >= klo && kg <= kmax) ? 0x0000ffffu : 0u) | ((kg + 1 >= klo && kg + 1 <= kmax) ? 0xffff0000u : 0u);
+    mhi = ((kg + 2 >= klo && kg + 2 <= kmax) ? 0x0000ffffu : 0u) | ((kg + 3 >= klo && kg + 3 <= kmax) ? 0xffff0000u : 0u);
+  }
+  bad = bad || (kg + 3 >= klo && kg <= kmax && !pagev_ok);
+}
+
+// The work on a tile whose keys are in ``kr``; its values are asked for first and used last.
+template <bool POW2>
+__device__ __forceinline__ void wp_work_tile(const WpGeom& G, int t0, int j, int qd, int lo, int pos, int klo, int kmax,
+                                             bool inner, float scale_log2, const s16x4 (&kr)[NSK], const s16x4 (&q)[NSK],
+                                             WpCol& c, f32x4 (&o)[NSV], bool& bad) {
+  uint2 v[NSV];
+  uint32_t mlo, mhi;
+  wp_load_v<POW2>(G, t0, j, qd, klo, kmax, inner, v, mlo, mhi, bad);
+  f32x4 s = (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int st = 0; st < NSK; ++st) s = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(kr[st], q[st], s, 0, 0, 0);
+  const int kg = t0 + 4 * qd;
+  bool ok[4];
+#pragma unroll
+  for (int r = 0; r < 4; ++r) ok[r] = inner || (kg + r <= pos && kg + r >= lo);
+  const s16x4 pw = wp_softmax_step(s, ok, scale_log2, c, o);
+#pragma unroll
+  for (int n = 0; n < NSV; ++n)
+    o[n] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(wp_s16x4(v[n].x & mlo, v[n].y & mhi), pw, o[n], 0, 0, 0);
+}
+
 // The tiles first, first + step, ... up to the one that holds key kmax, each tile's loads asked for a tile ahead.
 // CT: query heads of one key/value head that the wave takes for its rows; a tile that was loaded serves them all.
 // AHEAD false: no tile is asked for ahead.
 template <bool POW2, int CT, bool AHEAD>
 __device__ __forceinline__ void wp_walk_keys(const WpGeom& G, int first, int step, int j, int qd, int lo, int pos, int klo,
                                              int kmax, float scale_log2, const s16x4 (&q)[CT][NSK], WpCol (&c)[CT],
-                                             f32x4 (&o)[CT][NSV], bool& bad) {
+                                             f32x4 (&o)[CT][NSV], bool& bad, int inner_lo = 0x7fffffff, int inner_hi = -1) {
   if (first > kmax) return;
   if (!AHEAD) {                  // a tile's loads and its work in turn: fewer registers, so more waves share a SIMD
+    // inner_lo .. inner_hi: the keys that every column sees (tiles inside them take the short way)
+    const bool whole_pages = (G.ps & 15) == 0;
     for (int t0 = first; t0 <= kmax; t0 += step) {
-      WpKeys A;
-      wp_load_keys<POW2>(G, t0, j, qd, klo, kmax, A, bad);
+      const bool inner = whole_pages && t0 >= inner_lo && t0 + 15 <= inner_hi;
+      s16x4 kr[NSK];
+      wp_load_k<POW2>(G, t0, j, qd, klo, kmax, inner, kr, bad);
 #pragma unroll
-      for (int u = 0; u < CT; ++u) wp_use_keys(A, t0, qd, lo, pos, scale_log2, q[u], c[u], o[u]);
+      for (int u = 0; u < CT; ++u)
+        wp_work_tile<POW2>(G, t0, j, qd, lo, pos, klo, kmax, inner, scale_log2, kr, q[u], c[u], o[u], bad);
     }
     return;
   }
@@ -322,7 +401,10 @@ __global__ __launch_bounds__(256) void wpa_prefill_kernel(
   const int block_tiles = (nbmax + 15) / 16;
   for (int i = wave; i < block_tiles; i += 4) wp_tile_blocks<POW2>(G, i * 16, j, qd, nb, nbmax, scale_log2, qr, c, o, bad);
   const int turn = (wave + 4 - block_tiles % 4) % 4;
-  wp_walk_keys<POW2, 1, false>(G, (klo / 16 + turn) * 16, 64, j, qd, lo, pos, klo, kmax, scale_log2, qr1, c1, o1, bad);
+  // every column sees the keys from the last row's first key to the first row's own (when all 16 rows are there)
+  const bool all_rows = rb + 15 < qlen;
+  wp_walk_keys<POW2, 1, false>(G, (klo / 16 + turn) * 16, 64, j, qd, lo, pos, klo, kmax, scale_log2, qr1, c1, o1, bad,
+                               all_rows ? wp_first_key(kmax, window) : 0x7fffffff, all_rows ? ctx + rb : -1);
   // ---- the waves meet: a common maximum, then sums in the order of the waves
   if (qd == 0) s_m[wave][j] = c.m;
   __syncthreads();
